@@ -1,0 +1,127 @@
+/*
+ * splitwise_mixers.h -- C ABI of libsplitwise_mixers.so (gfx950 / MI355X).
+ *
+ * Operators of decoders that mix tokens by other means than rotary softmax attention over a full
+ * context: recurrent delta-rule layers with a per-sequence state, short causal convolutions,
+ * attention over a sliding window plus kept first tokens with the heads' weights mixed after the
+ * softmax, and norms with a single gain.  A library of its own so that a model that needs only
+ * these compiles only these.
+ *
+ * A step is a RAGGED batch: the new tokens of all sequences back to back in one token dimension.
+ *   q_start[B + 1]   first row of every sequence's tokens (int32, ascending, q_start[B] = rows)
+ *   ctx_len[B]       tokens of the sequence that earlier steps have run (its first new token's position)
+ *   token_seq[rows]  sequence index of every row
+ *   state_slot[B]    slot of the sequence in the recurrent-state pools
+ *   block_tables[B, table_width]   pages of the sequence in the paged caches
+ * A sequence with ctx_len == 0 starts from the empty state whatever its slot holds.
+ *
+ * Conventions as in splitwise_hip.h: SW_OK / negative status, swm_last_error(), asynchronous
+ * launches on `stream`, borrowed tensors.  `act_dtype` is SW_F32 or SW_BF16; everything that the
+ * comments call fp32 is fp32 in both.
+ */
+#ifndef SPLITWISE_MIXERS_H_
+#define SPLITWISE_MIXERS_H_
+
+#include <stdint.h>
+
+#include "splitwise_hip.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SWM_ABI_VERSION 1
+int swm_abi_version(void);
+const char* swm_last_error(void);
+
+/* residual[t] += y[t] / sqrt(mean(y[t]^2) + eps) * gain[0]   (residual fp32, y of y_dtype, gain fp32)
+ * and, when `cast_out` is not NULL, cast_out[t] = act_dtype(residual[t]). */
+int swm_scalar_norm_add(float* residual, const void* y, const float* gain, float eps, void* cast_out,
+                        int64_t rows, int width, int64_t y_stride, int y_dtype, int act_dtype, void* stream);
+/* out[t] = act_dtype(x[t] / sqrt(mean(x[t]^2) + eps) * gain[0]), x fp32. */
+int swm_scalar_norm(void* out, const float* x, const float* gain, float eps, int64_t rows, int width,
+                    int act_dtype, void* stream);
+
+/* Query / key norm over the WHOLE projection and the cache write of one attention layer.
+ * q_out[t] (fp32, [rows, q_size]) = q[t] / sqrt(mean(q[t]^2) + eps) * q_gain.  With k != NULL:
+ * key_cache[slot] = k[t] / sqrt(mean(k[t]^2) + eps) * k_gain and value_cache[slot] = v[t], where
+ * slot = slot_mapping[t] (int64, < 0: row not cached); caches are [slots, k_size] / [slots, v_size]
+ * in act_dtype. */
+int swm_qk_norm_cache(float* q_out, const void* q, const void* k, const void* v, int64_t in_stride,
+                      const float* q_gain, const float* k_gain, float eps, void* key_cache, void* value_cache,
+                      const int64_t* slot_mapping, int64_t rows, int q_size, int k_size, int v_size,
+                      int act_dtype, void* stream);
+
+/* Attention of every new token over its sequence's paged keys: position i sees j <= i with
+ * i - j < window or j < keep_first; softmax over those; then head h's weights become
+ * sum_g talk[h, g] * weights_g and are applied to the values of h's own key/value head.
+ * q fp32 [rows, heads * dim]; caches [pages * page_size, kv_heads * dim | vdim] act_dtype;
+ * talk fp32 [heads, heads]; out act_dtype [rows, heads * vdim].
+ * `tiled` != 0 picks the kernel that shares staged keys among 16 consecutive queries of a sequence
+ * (prompt portions); 0 the one-token-per-workgroup kernel (decode steps). */
+int swm_window_attention(void* out, const float* q, const void* key_cache, const void* value_cache,
+                         const float* talk, const int32_t* block_tables, int table_width,
+                         const int32_t* q_start, const int32_t* ctx_len, const int32_t* token_seq,
+                         int64_t rows, int num_seqs, int heads, int kv_heads, int dim, int vdim, int page_size,
+                         float scale, int window, int keep_first, int tiled, int act_dtype, void* stream);
+
+/* Short causal convolution over time per channel, then silu.  x act_dtype [rows, channels] (row stride
+ * x_stride); taps fp32 [channels, num_taps], last column = current token; state fp32
+ * [slots, num_taps - 1, channels] = the sequence's last num_taps - 1 inputs; out fp32 [rows, channels].
+ * swm_short_conv reads the state; swm_short_conv_advance then moves it past the step's tokens. */
+int swm_short_conv(float* out, const void* x, int64_t x_stride, const float* taps, const float* state,
+                   const int32_t* q_start, const int32_t* ctx_len, const int32_t* token_seq,
+                   const int32_t* state_slot, int64_t rows, int channels, int num_taps, int act_dtype,
+                   void* stream);
+int swm_short_conv_advance(float* state, const void* x, int64_t x_stride, const int32_t* q_start,
+                           const int32_t* ctx_len, const int32_t* state_slot, int num_seqs, int channels,
+                           int num_taps, int act_dtype, void* stream);
+
+/* Delta rule with a gate and a decay per head and key channel, token by token per sequence:
+ *   S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
+ * with q, k made unit vectors per head (eps 1e-6 inside the root; q also times dim^-1/2),
+ * beta = sigmoid(beta_pre), g = exp(-exp(a_log[head]) * softplus(decay_pre + dt_bias)).
+ * qkv fp32 [rows, 2 * kv_heads * dim + heads * vdim] (q | k | v after the short convolution);
+ * beta_pre act_dtype [rows, heads] (row stride beta_stride); decay_pre act_dtype [rows, heads * dim];
+ * dt_bias fp32 [heads * dim]; a_log fp32 [heads]; state fp32 [slots, heads, dim, vdim];
+ * out fp32 [rows, heads * vdim]. */
+int swm_channel_delta(float* out, const float* qkv, const void* beta_pre, int64_t beta_stride,
+                      const void* decay_pre, const float* dt_bias, const float* a_log, float* state,
+                      const int32_t* q_start, const int32_t* ctx_len, const int32_t* state_slot,
+                      int num_seqs, int heads, int kv_heads, int dim, int vdim, int act_dtype, void* stream);
+
+/* Delta rule with a decay and a removal rate per head and key channel:
+ *   S <- diag(w) S - (a * u) (u^T S) + k v^T   (both terms read the old S);  o = S^T r
+ * u = k / sqrt(sum k^2 + 1e-6), w = exp(-exp(-1/2) sigmoid(decay_pre + w0)), a = sigmoid(rate_pre + a_bias).
+ * r, k, v act_dtype [rows, heads * dim] (row stride rkv_stride); decay_pre, rate_pre act_dtype
+ * [rows, heads * dim] (row strides given); w0, a_bias fp32 [heads * dim]; state fp32 [slots, heads, dim, dim];
+ * out fp32 [rows, heads * dim]. */
+int swm_general_delta(float* out, const void* r, const void* k, const void* v, int64_t rkv_stride,
+                      const void* decay_pre, int64_t decay_stride, const float* w0, const void* rate_pre,
+                      int64_t rate_stride, const float* a_bias, float* state, const int32_t* q_start,
+                      const int32_t* ctx_len, const int32_t* state_slot, int num_seqs, int heads, int dim,
+                      int act_dtype, void* stream);
+
+/* out[t, h, :] = act_dtype(o / sqrt(mean(o^2) + eps) * weight[h * weight_head_stride + :] * sigmoid(gate[t, h, :]))
+ * o fp32 [rows, heads * vdim]; gate act_dtype (row stride gate_stride); weight fp32. */
+int swm_head_norm_gate(void* out, const float* o, const void* gate, int64_t gate_stride, const float* weight,
+                       int weight_head_stride, float eps, int64_t rows, int heads, int vdim, int act_dtype,
+                       void* stream);
+
+/* Feed-forward experts over (row, choice) pairs sorted by expert: `order` (int32 [pairs]) holds
+ * row * top + choice of every sorted pair and expert e owns the sorted pairs
+ * [expert_start[e], expert_start[e + 1]).
+ * hidden[pair] = gelu_erf(up[e] x[order[pair] / top])   (act_dtype [pairs, ff]; up act_dtype [experts, ff, width]) */
+int swm_expert_up_gelu(void* hidden, const void* x, const void* up, const int32_t* order,
+                       const int32_t* expert_start, int num_experts, int64_t sorted_rows, int width, int ff,
+                       int top, int act_dtype, void* stream);
+/* out[order[pair] / top] += weight * down[e] hidden[pair]   (out fp32 [rows, width], zeroed by the caller;
+ * down act_dtype [experts, width, ff]; atomic adds when top > 1). */
+int swm_expert_down(float* out, const void* hidden, const void* down, const int32_t* order,
+                    const int32_t* expert_start, int num_experts, int64_t sorted_rows, int width, int ff,
+                    int top, float weight, int act_dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

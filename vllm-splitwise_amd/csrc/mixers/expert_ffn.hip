@@ -1,0 +1,166 @@
+// Feed-forward experts over rows that were sorted by expert: two grouped "NT" GEMMs (both operands
+// contiguous along the reduction), the first with the exact gelu as its epilogue, the second scattering
+// its rows back and adding them into an fp32 output.
+//
+// The host does not know how many rows an expert got (the sort stays on the device), so the grid has the
+// upper bound ceil(pairs / TM) + experts row tiles and each workgroup finds its (expert, tile) from the
+// prefix sums; surplus workgroups leave at once.  Tiles never straddle two experts.
+#include "mixers_common.cuh"
+
+namespace swm {
+
+constexpr int TM = 32, TN = 64, TK = 32, kFfnThreads = 256;
+
+__device__ __forceinline__ float gelu_erf(float z) { return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f)); }
+
+// -> expert and first sorted row of this workgroup's tile, rows in it (0: nothing to do)
+__device__ __forceinline__ int find_tile(const int32_t* __restrict__ expert_start, int num_experts, int tile,
+                                         int* expert, int* row0) {
+  for (int e = 0; e < num_experts; ++e) {
+    const int lo = expert_start[e], n = expert_start[e + 1] - lo;
+    const int tiles = (n + TM - 1) / TM;
+    if (tile < tiles) {
+      *expert = e;
+      *row0 = lo + tile * TM;
+      return min(TM, n - tile * TM);
+    }
+    tile -= tiles;
+  }
+  return 0;
+}
+
+// acc[2][4] of thread (ty, tx): rows 2 * ty + {0, 1}, columns tx + 16 * {0..3} of the tile
+//   A row p: a_base + a_row(p) * K        B row n: b_base + n * K
+template <typename T, typename RowOf>
+__device__ __forceinline__ void tile_gemm(float (&acc)[2][4], const void* __restrict__ a, RowOf a_row, int rows,
+                                          const void* __restrict__ b, int64_t b_off, int n0, int N, int K,
+                                          float (*As)[TK + 1], float (*Bs)[TK + 1]) {
+  const int tid = threadIdx.x, ty = tid >> 4, tx = tid & 15;
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = 0.0f;
+  for (int k0 = 0; k0 < K; k0 += TK) {
+    // A tile: 32 x 32 = 1024 values, 4 per thread; B tile: 64 x 32 = 2048 values, 8 per thread
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+      const int e = tid + it * kFfnThreads, r = e >> 5, k = e & 31;
+      float v = 0.0f;
+      if (r < rows && k0 + k < K) v = ld<T>(a, a_row(r) * (int64_t)K + k0 + k);
+      As[r][k] = v;
+    }
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+      const int e = tid + it * kFfnThreads, r = e >> 5, k = e & 31;
+      float v = 0.0f;
+      if (n0 + r < N && k0 + k < K) v = ld<T>(b, b_off + (int64_t)(n0 + r) * K + k0 + k);
+      Bs[r][k] = v;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < TK; ++k) {
+      const float a0 = As[2 * ty][k], a1 = As[2 * ty + 1][k];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float bv = Bs[tx + 16 * j][k];
+        acc[0][j] += a0 * bv;
+        acc[1][j] += a1 * bv;
+      }
+    }
+    __syncthreads();
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kFfnThreads) void expert_up_gelu_kernel(
+    void* __restrict__ hidden, const void* __restrict__ x, const void* __restrict__ up,
+    const int32_t* __restrict__ order, const int32_t* __restrict__ expert_start, int num_experts, int width, int ff,
+    int top) {
+  __shared__ float As[TM][TK + 1];
+  __shared__ float Bs[TN][TK + 1];
+  int e, row0;
+  const int rows = find_tile(expert_start, num_experts, blockIdx.x, &e, &row0);
+  if (rows == 0) return;
+  const int n0 = blockIdx.y * TN;
+  float acc[2][4];
+  tile_gemm<T>(acc, x, [&](int r) { return (int64_t)(order[row0 + r] / top); }, rows, up, (int64_t)e * ff * width, n0, ff,
+               width, As, Bs);
+  const int ty = threadIdx.x >> 4, tx = threadIdx.x & 15;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int r = 2 * ty + i;
+    if (r >= rows) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + tx + 16 * j;
+      if (n < ff) st<T>(hidden, (int64_t)(row0 + r) * ff + n, gelu_erf(acc[i][j]));
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kFfnThreads) void expert_down_kernel(
+    float* __restrict__ out, const void* __restrict__ hidden, const void* __restrict__ down,
+    const int32_t* __restrict__ order, const int32_t* __restrict__ expert_start, int num_experts, int width, int ff,
+    int top, float weight) {
+  __shared__ float As[TM][TK + 1];
+  __shared__ float Bs[TN][TK + 1];
+  int e, row0;
+  const int rows = find_tile(expert_start, num_experts, blockIdx.x, &e, &row0);
+  if (rows == 0) return;
+  const int n0 = blockIdx.y * TN;
+  float acc[2][4];
+  tile_gemm<T>(acc, hidden, [&](int r) { return (int64_t)(row0 + r); }, rows, down, (int64_t)e * width * ff, n0, width,
+               ff, As, Bs);
+  const int ty = threadIdx.x >> 4, tx = threadIdx.x & 15;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int r = 2 * ty + i;
+    if (r >= rows) continue;
+    const int64_t dst = order[row0 + r] / top;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + tx + 16 * j;
+      if (n >= width) continue;
+      float* p = out + dst * width + n;
+      if (top == 1) *p += weight * acc[i][j];           // a row has one expert: nobody else writes it
+      else atomicAdd(p, weight * acc[i][j]);
+    }
+  }
+}
+
+}  // namespace swm
+
+extern "C" {
+
+int swm_expert_up_gelu(void* hidden, const void* x, const void* up, const int32_t* order,
+                       const int32_t* expert_start, int num_experts, int64_t sorted_rows, int width, int ff,
+                       int top, int act_dtype, void* stream) {
+  using namespace swm;
+  if (sorted_rows == 0) return SW_OK;
+  SW_CHECK_ARG(act_ok(act_dtype), "expert_up_gelu: unsupported dtype %d", act_dtype);
+  SW_CHECK_ARG(num_experts > 0 && width > 0 && ff > 0 && top > 0 && sorted_rows < (1ll << 30), "expert_up_gelu: bad shape");
+  const dim3 grid((unsigned)((sorted_rows + TM - 1) / TM + num_experts), (unsigned)((ff + TN - 1) / TN));
+  SWM_DISPATCH_ACT(act_dtype, hipLaunchKernelGGL(expert_up_gelu_kernel<T>, grid, dim3(kFfnThreads), 0,
+                                                 static_cast<hipStream_t>(stream), hidden, x, up, order, expert_start,
+                                                 num_experts, width, ff, top););
+  SW_CHECK_LAUNCH();
+  return SW_OK;
+}
+
+int swm_expert_down(float* out, const void* hidden, const void* down, const int32_t* order,
+                    const int32_t* expert_start, int num_experts, int64_t sorted_rows, int width, int ff,
+                    int top, float weight, int act_dtype, void* stream) {
+  using namespace swm;
+  if (sorted_rows == 0) return SW_OK;
+  SW_CHECK_ARG(act_ok(act_dtype), "expert_down: unsupported dtype %d", act_dtype);
+  SW_CHECK_ARG(num_experts > 0 && width > 0 && ff > 0 && top > 0 && sorted_rows < (1ll << 30), "expert_down: bad shape");
+  const dim3 grid((unsigned)((sorted_rows + TM - 1) / TM + num_experts), (unsigned)((width + TN - 1) / TN));
+  SWM_DISPATCH_ACT(act_dtype, hipLaunchKernelGGL(expert_down_kernel<T>, grid, dim3(kFfnThreads), 0,
+                                                 static_cast<hipStream_t>(stream), out, hidden, down, order,
+                                                 expert_start, num_experts, width, ff, top, weight););
+  SW_CHECK_LAUNCH();
+  return SW_OK;
+}
+
+}  // extern "C"

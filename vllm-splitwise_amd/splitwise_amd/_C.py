@@ -833,3 +833,8 @@ kv_ops = SimpleNamespace(
 cuda_utils = SimpleNamespace(
     get_max_shared_memory_per_block_device_attribute=get_max_shared_memory_per_block_device_attribute,
 )
+
+# operators of recurrent / windowed token mixers live in a library of their own (built by `make mixers`)
+from . import _C_mixers  # noqa: E402
+
+mixer_ops = _C_mixers.ops

@@ -1,0 +1,320 @@
+"""ctypes binding of libsplitwise_mixers.so: the operators of recurrent / windowed token mixers
+(``include/splitwise_mixers.h``).  Same rules as ``_C``: raw device pointers, torch's current HIP
+stream, RuntimeError when the library is missing or an entry point refuses its arguments; no fallback.
+
+Every operator takes the step's ragged layout as a ``RaggedBatch``-like object with the int32 device
+tensors ``q_start`` [B + 1], ``ctx_len`` [B], ``token_seq`` [rows], ``state_slot`` [B] and
+``block_tables`` [B, width].
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+from types import SimpleNamespace
+from typing import Optional
+
+import torch
+
+_PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_PKG_DIR, "libsplitwise_mixers.so")
+ABI_VERSION = 1
+
+SW_F32, SW_BF16 = 0, 2
+_ACT = {torch.float32: SW_F32, torch.bfloat16: SW_BF16}
+
+_p, _i, _l, _f = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_float
+_SIGNATURES = {
+    "swm_scalar_norm_add": [_p, _p, _p, _f, _p, _l, _i, _l, _i, _i, _p],
+    "swm_scalar_norm": [_p, _p, _p, _f, _l, _i, _i, _p],
+    "swm_qk_norm_cache": [_p, _p, _p, _p, _l, _p, _p, _f, _p, _p, _p, _l, _i, _i, _i, _i, _p],
+    "swm_window_attention": [_p, _p, _p, _p, _p, _p, _i, _p, _p, _p, _l, _i, _i, _i, _i, _i, _i, _f, _i, _i, _i,
+                             _i, _p],
+    "swm_short_conv": [_p, _p, _l, _p, _p, _p, _p, _p, _p, _l, _i, _i, _i, _p],
+    "swm_short_conv_advance": [_p, _p, _l, _p, _p, _p, _i, _i, _i, _i, _p],
+    "swm_channel_delta": [_p, _p, _p, _l, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p],
+    "swm_general_delta": [_p, _p, _p, _p, _l, _p, _l, _p, _p, _l, _p, _p, _p, _p, _p, _i, _i, _i, _i, _p],
+    "swm_head_norm_gate": [_p, _p, _p, _l, _p, _i, _f, _l, _i, _i, _i, _p],
+    "swm_expert_up_gelu": [_p, _p, _p, _p, _p, _i, _l, _i, _i, _i, _i, _p],
+    "swm_expert_down": [_p, _p, _p, _p, _p, _i, _l, _i, _i, _i, _f, _i, _p],
+}
+
+_lib = None
+
+
+def library_path() -> str:
+    return _LIB_PATH
+
+
+def build_library() -> None:
+    """Compiles only this library (``make mixers``): what a fresh checkout needs before its first step."""
+    subprocess.run(["make", "-C", os.path.dirname(_PKG_DIR), "mixers", "-j", str(min(8, os.cpu_count() or 1))],
+                   check=True, stdout=subprocess.DEVNULL)
+
+
+def load_library() -> ctypes.CDLL:
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(_LIB_PATH):
+        raise RuntimeError(f"native library not built: {_LIB_PATH} is missing (run `make -C vllm-splitwise_amd mixers`)")
+    lib = ctypes.CDLL(_LIB_PATH)
+    lib.swm_last_error.restype, lib.swm_last_error.argtypes = ctypes.c_char_p, []
+    lib.swm_abi_version.restype, lib.swm_abi_version.argtypes = _i, []
+    if lib.swm_abi_version() != ABI_VERSION:
+        raise RuntimeError(f"{_LIB_PATH} implements interface version {lib.swm_abi_version()}, this binding needs "
+                           f"{ABI_VERSION}: rebuild it (`make -C vllm-splitwise_amd mixers`)")
+    for name, argtypes in _SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.argtypes, fn.restype = argtypes, _i
+    _lib = lib
+    return lib
+
+
+def _check(status: int) -> None:
+    if status != 0:
+        raise RuntimeError(load_library().swm_last_error().decode("utf-8", "replace")
+                           or f"splitwise_mixers call failed with status {status}")
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _act(t: torch.Tensor) -> int:
+    try:
+        return _ACT[t.dtype]
+    except KeyError:
+        raise RuntimeError(f"Unsupported data type: {t.dtype}") from None
+
+
+def _need(cond: bool, what: str) -> None:
+    if not cond:
+        raise RuntimeError(what)
+
+
+def _dev(*tensors: Optional[torch.Tensor]) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("splitwise_mixers operators need tensors on a HIP device")
+
+
+def _f32c(t: torch.Tensor, what: str) -> None:
+    _need(t.dtype == torch.float32 and t.is_contiguous(), f"{what} must be a contiguous fp32 tensor")
+
+
+def _rows(t: torch.Tensor, what: str) -> int:
+    """Row stride (elements) of a 2-D view whose rows are contiguous."""
+    _need(t.dim() == 2 and t.stride(1) == 1, f"{what} must be 2-D with contiguous rows")
+    return t.stride(0)
+
+
+def scalar_norm_add(residual: torch.Tensor, y: torch.Tensor, gain: torch.Tensor, eps: float,
+                    cast_out: Optional[torch.Tensor] = None) -> None:
+    """residual (fp32, in place) += y / rms(y) * gain; cast_out = the new residual in cast_out's dtype."""
+    _dev(residual, y, gain, cast_out)
+    _f32c(residual, "residual")
+    _f32c(gain, "gain")
+    _need(residual.shape == y.shape and gain.numel() == 1, "scalar_norm_add: shapes")
+    stride = _rows(y, "y")
+    if cast_out is not None:
+        _need(cast_out.is_contiguous() and cast_out.shape == y.shape, "scalar_norm_add: cast_out")
+    with torch.cuda.device(y.device):
+        _check(load_library().swm_scalar_norm_add(
+            residual.data_ptr(), y.data_ptr(), gain.data_ptr(), eps,
+            None if cast_out is None else cast_out.data_ptr(), y.shape[0], y.shape[1], stride, _act(y),
+            _act(y if cast_out is None else cast_out), _stream(y)))
+
+
+def scalar_norm(out: torch.Tensor, x: torch.Tensor, gain: torch.Tensor, eps: float) -> None:
+    _dev(out, x, gain)
+    _f32c(x, "x")
+    _f32c(gain, "gain")
+    _need(out.is_contiguous() and out.shape == x.shape and x.dim() == 2 and gain.numel() == 1, "scalar_norm: shapes")
+    with torch.cuda.device(x.device):
+        _check(load_library().swm_scalar_norm(out.data_ptr(), x.data_ptr(), gain.data_ptr(), eps, x.shape[0],
+                                              x.shape[1], _act(out), _stream(x)))
+
+
+def qk_norm_cache(q_out: torch.Tensor, q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.Tensor],
+                  q_gain: torch.Tensor, k_gain: Optional[torch.Tensor], eps: float,
+                  key_cache: Optional[torch.Tensor], value_cache: Optional[torch.Tensor],
+                  slot_mapping: Optional[torch.Tensor]) -> None:
+    """q, k, v: column ranges of ONE projection output (same row stride).  Caches: [pages, page, kv * size]."""
+    _dev(q_out, q, k, v, q_gain, k_gain, key_cache, value_cache, slot_mapping)
+    _f32c(q_out, "q_out")
+    _f32c(q_gain, "q_gain")
+    stride = _rows(q, "q")
+    rows, q_size = q.shape
+    _need(q_out.shape == q.shape and q_gain.numel() == q_size, "qk_norm_cache: query shapes")
+    k_size = v_size = 0
+    if k is not None:
+        _need(v is not None and k_gain is not None and key_cache is not None and value_cache is not None
+              and slot_mapping is not None, "qk_norm_cache: keys need values, a gain, caches and slots")
+        _f32c(k_gain, "k_gain")
+        k_size, v_size = k.shape[1], v.shape[1]
+        _need(_rows(k, "k") == stride and _rows(v, "v") == stride and k.dtype == q.dtype and v.dtype == q.dtype
+              and k.shape[0] == rows and v.shape[0] == rows, "qk_norm_cache: q, k, v must share rows and stride")
+        _need(k_gain.numel() == k_size and key_cache.dtype == q.dtype and value_cache.dtype == q.dtype
+              and key_cache.is_contiguous() and value_cache.is_contiguous()
+              and key_cache.shape[-1] == k_size and value_cache.shape[-1] == v_size, "qk_norm_cache: cache shapes")
+        _need(slot_mapping.dtype == torch.int64 and slot_mapping.numel() == rows and slot_mapping.is_contiguous(),
+              "qk_norm_cache: slot_mapping must be int64 [rows]")
+        slots = key_cache.shape[0] * key_cache.shape[1]
+        _need(value_cache.shape[0] * value_cache.shape[1] == slots, "qk_norm_cache: caches differ in slots")
+    with torch.cuda.device(q.device):
+        _check(load_library().swm_qk_norm_cache(
+            q_out.data_ptr(), q.data_ptr(), None if k is None else k.data_ptr(), None if v is None else v.data_ptr(),
+            stride, q_gain.data_ptr(), None if k is None else k_gain.data_ptr(), eps,
+            None if k is None else key_cache.data_ptr(), None if k is None else value_cache.data_ptr(),
+            None if k is None else slot_mapping.data_ptr(), rows, q_size, k_size, v_size, _act(q), _stream(q)))
+
+
+def _ragged_ok(batch, rows: int) -> int:
+    n = batch.ctx_len.numel()
+    for name in ("q_start", "ctx_len", "token_seq", "state_slot"):
+        t = getattr(batch, name)
+        _need(t is not None and t.dtype == torch.int32 and t.is_contiguous() and t.is_cuda, f"ragged batch: {name}")
+    _need(batch.q_start.numel() == n + 1 and batch.token_seq.numel() == rows and batch.state_slot.numel() == n,
+          "ragged batch: lengths")
+    return n
+
+
+def window_attention(out: torch.Tensor, q: torch.Tensor, key_cache: torch.Tensor, value_cache: torch.Tensor,
+                     talk: torch.Tensor, batch, heads: int, kv_heads: int, dim: int, vdim: int, scale: float,
+                     window: int, keep_first: int, tiled: bool = False) -> None:
+    """out [rows, heads * vdim] (cache dtype); q fp32 [rows, heads * dim]; caches [pages, page, kv_heads * size]."""
+    _dev(out, q, key_cache, value_cache, talk)
+    _f32c(q, "q")
+    _f32c(talk, "talk")
+    rows = q.shape[0]
+    n = _ragged_ok(batch, rows)
+    tables = batch.block_tables
+    _need(tables.dtype == torch.int32 and tables.is_contiguous() and tables.dim() == 2 and tables.shape[0] == n,
+          "window_attention: block tables")
+    _need(q.shape[1] == heads * dim and out.shape == (rows, heads * vdim) and out.is_contiguous()
+          and out.dtype == key_cache.dtype == value_cache.dtype and talk.shape == (heads, heads)
+          and key_cache.is_contiguous() and value_cache.is_contiguous()
+          and key_cache.shape[1:] == (value_cache.shape[1], kv_heads * dim)
+          and value_cache.shape[2] == kv_heads * vdim and key_cache.shape[0] == value_cache.shape[0],
+          "window_attention: shapes")
+    _need(batch.max_pages_used <= tables.shape[1] and batch.max_page_id < key_cache.shape[0],
+          "window_attention: block tables exceed the cache")
+    with torch.cuda.device(q.device):
+        _check(load_library().swm_window_attention(
+            out.data_ptr(), q.data_ptr(), key_cache.data_ptr(), value_cache.data_ptr(), talk.data_ptr(),
+            tables.data_ptr(), tables.shape[1], batch.q_start.data_ptr(), batch.ctx_len.data_ptr(),
+            batch.token_seq.data_ptr(), rows, n, heads, kv_heads, dim, vdim, key_cache.shape[1], scale, window,
+            keep_first, int(tiled), _act(out), _stream(q)))
+
+
+def short_conv(out: torch.Tensor, x: torch.Tensor, taps: torch.Tensor, state: torch.Tensor, batch) -> None:
+    """out fp32 [rows, channels] = silu(causal conv of x with the sequence's carried inputs); the state
+    [slots, taps - 1, channels] is read here and moved on by ``short_conv_advance``."""
+    _dev(out, x, taps, state)
+    _f32c(out, "out")
+    _f32c(taps, "taps")
+    _f32c(state, "state")
+    stride = _rows(x, "x")
+    rows, channels = x.shape
+    n = _ragged_ok(batch, rows)
+    k = taps.shape[1]
+    _need(out.shape == x.shape and taps.shape[0] == channels and state.shape[1:] == (k - 1, channels)
+          and batch.max_state_slot < state.shape[0], "short_conv: shapes")
+    with torch.cuda.device(x.device):
+        lib = load_library()
+        _check(lib.swm_short_conv(out.data_ptr(), x.data_ptr(), stride, taps.data_ptr(), state.data_ptr(),
+                                  batch.q_start.data_ptr(), batch.ctx_len.data_ptr(), batch.token_seq.data_ptr(),
+                                  batch.state_slot.data_ptr(), rows, channels, k, _act(x), _stream(x)))
+        _check(lib.swm_short_conv_advance(state.data_ptr(), x.data_ptr(), stride, batch.q_start.data_ptr(),
+                                          batch.ctx_len.data_ptr(), batch.state_slot.data_ptr(), n, channels, k,
+                                          _act(x), _stream(x)))
+
+
+def channel_delta(out: torch.Tensor, qkv: torch.Tensor, beta_pre: torch.Tensor, decay_pre: torch.Tensor,
+                  dt_bias: torch.Tensor, a_log: torch.Tensor, state: torch.Tensor, batch, heads: int, kv_heads: int,
+                  dim: int, vdim: int) -> None:
+    _dev(out, qkv, beta_pre, decay_pre, dt_bias, a_log, state)
+    for t, what in ((out, "out"), (qkv, "qkv"), (dt_bias, "dt_bias"), (a_log, "a_log"), (state, "state")):
+        _f32c(t, what)
+    rows = qkv.shape[0]
+    n = _ragged_ok(batch, rows)
+    _need(qkv.shape[1] == 2 * kv_heads * dim + heads * vdim and out.shape == (rows, heads * vdim)
+          and beta_pre.shape == (rows, heads) and decay_pre.shape == (rows, heads * dim) and decay_pre.is_contiguous()
+          and decay_pre.dtype == beta_pre.dtype and dt_bias.numel() == heads * dim and a_log.numel() == heads
+          and state.shape[1:] == (heads, dim, vdim) and batch.max_state_slot < state.shape[0],
+          "channel_delta: shapes")
+    with torch.cuda.device(qkv.device):
+        _check(load_library().swm_channel_delta(
+            out.data_ptr(), qkv.data_ptr(), beta_pre.data_ptr(), _rows(beta_pre, "beta_pre"), decay_pre.data_ptr(),
+            dt_bias.data_ptr(), a_log.data_ptr(), state.data_ptr(), batch.q_start.data_ptr(),
+            batch.ctx_len.data_ptr(), batch.state_slot.data_ptr(), n, heads, kv_heads, dim, vdim, _act(decay_pre),
+            _stream(qkv)))
+
+
+def general_delta(out: torch.Tensor, r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay_pre: torch.Tensor,
+                  w0: torch.Tensor, rate_pre: torch.Tensor, a_bias: torch.Tensor, state: torch.Tensor, batch,
+                  heads: int, dim: int) -> None:
+    _dev(out, r, k, v, decay_pre, w0, rate_pre, a_bias, state)
+    for t, what in ((out, "out"), (w0, "w0"), (a_bias, "a_bias"), (state, "state")):
+        _f32c(t, what)
+    rows = r.shape[0]
+    n = _ragged_ok(batch, rows)
+    stride = _rows(r, "r")
+    size = heads * dim
+    _need(all(t.shape == (rows, size) and t.dtype == r.dtype for t in (r, k, v, decay_pre, rate_pre))
+          and _rows(k, "k") == stride and _rows(v, "v") == stride and out.shape == (rows, size)
+          and w0.numel() == size and a_bias.numel() == size and state.shape[1:] == (heads, dim, dim)
+          and batch.max_state_slot < state.shape[0], "general_delta: shapes")
+    with torch.cuda.device(r.device):
+        _check(load_library().swm_general_delta(
+            out.data_ptr(), r.data_ptr(), k.data_ptr(), v.data_ptr(), stride, decay_pre.data_ptr(),
+            _rows(decay_pre, "decay_pre"), w0.data_ptr(), rate_pre.data_ptr(), _rows(rate_pre, "rate_pre"),
+            a_bias.data_ptr(), state.data_ptr(), batch.q_start.data_ptr(), batch.ctx_len.data_ptr(),
+            batch.state_slot.data_ptr(), n, heads, dim, _act(r), _stream(r)))
+
+
+def head_norm_gate(out: torch.Tensor, o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, per_head_weight: bool,
+                   eps: float, heads: int, vdim: int) -> None:
+    """``per_head_weight``: weight is [heads * vdim]; otherwise [vdim], shared by the heads."""
+    _dev(out, o, gate, weight)
+    _f32c(o, "o")
+    _f32c(weight, "weight")
+    rows = o.shape[0]
+    _need(o.shape == (rows, heads * vdim) and gate.shape == o.shape and out.shape == o.shape and out.is_contiguous()
+          and out.dtype == gate.dtype and weight.numel() == (heads * vdim if per_head_weight else vdim),
+          "head_norm_gate: shapes")
+    with torch.cuda.device(o.device):
+        _check(load_library().swm_head_norm_gate(out.data_ptr(), o.data_ptr(), gate.data_ptr(), _rows(gate, "gate"),
+                                                 weight.data_ptr(), vdim if per_head_weight else 0, eps, rows, heads,
+                                                 vdim, _act(out), _stream(o)))
+
+
+def expert_ffn(out: torch.Tensor, x: torch.Tensor, up: torch.Tensor, down: torch.Tensor, order: torch.Tensor,
+               expert_start: torch.Tensor, top: int, weight: float) -> None:
+    """out (fp32 [rows, width], zeroed by the caller) += weight * sum over each row's experts of
+    down[e] gelu(up[e] x[row]); ``order`` / ``expert_start`` as ``TableRoutedExperts.route`` makes them."""
+    _dev(out, x, up, down, order, expert_start)
+    _f32c(out, "out")
+    rows, width = x.shape
+    experts, ff = up.shape[0], up.shape[1]
+    _need(x.is_contiguous() and up.is_contiguous() and down.is_contiguous() and up.dtype == x.dtype == down.dtype
+          and up.shape == (experts, ff, width) and down.shape == (experts, width, ff) and out.shape == (rows, width)
+          and order.dtype == torch.int32 and order.numel() == rows * top and order.is_contiguous()
+          and expert_start.dtype == torch.int32 and expert_start.numel() == experts + 1
+          and expert_start.is_contiguous(), "expert_ffn: shapes")
+    pairs = rows * top
+    hidden = torch.empty(pairs, ff, dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        lib = load_library()
+        _check(lib.swm_expert_up_gelu(hidden.data_ptr(), x.data_ptr(), up.data_ptr(), order.data_ptr(),
+                                      expert_start.data_ptr(), experts, pairs, width, ff, top, _act(x), _stream(x)))
+        _check(lib.swm_expert_down(out.data_ptr(), hidden.data_ptr(), down.data_ptr(), order.data_ptr(),
+                                   expert_start.data_ptr(), experts, pairs, width, ff, top, weight, _act(x),
+                                   _stream(x)))
+
+
+ops = SimpleNamespace(expert_ffn=expert_ffn, 
+    scalar_norm_add=scalar_norm_add, scalar_norm=scalar_norm, qk_norm_cache=qk_norm_cache,
+    window_attention=window_attention, short_conv=short_conv, channel_delta=channel_delta,
+    general_delta=general_delta, head_norm_gate=head_norm_gate)

@@ -87,6 +87,9 @@ class ModelConfig:
         if os.path.isfile(cfg_path):
             with open(cfg_path) as f:
                 raw = json.load(f)
+            if raw.get("architecture") == "Nepevik":
+                from .model_executor.models.nepevik import normalize_config
+                return normalize_config(raw)
             arch = (raw.get("architectures") or [""])[0].lower()
             raw["architecture"] = "opt" if "opt" in arch else "llama"
             raw.setdefault("num_key_value_heads", raw["num_attention_heads"])
@@ -123,6 +126,23 @@ class ModelConfig:
 
     def get_num_layers(self, parallel_config: "ParallelConfig") -> int:
         return self.hf_config["num_hidden_layers"] // parallel_config.pipeline_parallel_size
+
+    def model_class(self):
+        from .model_executor.model_loader import architecture_class
+        return architecture_class(self.architecture)
+
+    @property
+    def uses_ragged_steps(self) -> bool:
+        """Models whose layers carry a per-sequence state (or take prompts in portions) get every step in
+        the ragged layout; the scheduler then mixes prompt portions and decoded tokens in one step."""
+        return bool(getattr(self.model_class(), "uses_ragged_steps", False))
+
+    def get_cache_layout(self, block_size: int):
+        """Per-layer cache needs of a model that is not a stack of equal attention layers, else None."""
+        cls = self.model_class()
+        if hasattr(cls, "cache_layout"):
+            return cls.cache_layout(self.hf_config, block_size)
+        return None
 
 
 class CacheConfig:
@@ -191,7 +211,10 @@ class SchedulerConfig:
 
     def __init__(self, max_num_batched_tokens: Optional[int], max_num_seqs: int, max_model_len: int,
                  max_paddings: int = 256, prefill_batch_tokens: int = 0, prefill_max_wait: float = 0.1,
-                 pipeline_steps: bool = False) -> None:
+                 pipeline_steps: bool = False, ragged_steps: bool = False) -> None:
+        # ragged steps: a step mixes portions of prompts (cut to the token budget) with decoded tokens, and
+        # every live sequence owns one of ``max_num_seqs`` recurrent-state slots
+        self.ragged_steps = ragged_steps
         # prefill batching (0 = off: prompts are admitted as soon as they fit, as in the reference)
         self.prefill_batch_tokens = prefill_batch_tokens
         self.pipeline_steps = pipeline_steps
@@ -202,7 +225,7 @@ class SchedulerConfig:
         self.max_num_seqs = max_num_seqs
         self.max_model_len = max_model_len
         self.max_paddings = max_paddings
-        if self.max_num_batched_tokens < self.max_model_len:
+        if self.max_num_batched_tokens < self.max_model_len and not ragged_steps:
             raise ValueError(f"max_num_batched_tokens ({self.max_num_batched_tokens}) is smaller than "
                              f"max_model_len ({self.max_model_len}).")
         if self.max_num_batched_tokens < self.max_num_seqs:

@@ -306,6 +306,20 @@ class BlockSpaceManager:
         self.gpu_allocator.free(last)
         return last, fresh
 
+    # --------------------------------------------------------- growing by several tokens
+    def blocks_missing(self, seq: Sequence) -> int:
+        """Blocks that ``extend`` would have to take for the sequence's tokens as they are now."""
+        return max(0, seq.num_logical_blocks - len(self.block_tables.get(seq.seq_id, ())))
+
+    def extend(self, seq: Sequence) -> None:
+        """Ragged steps: room for every token of the sequence, however many were appended since the last
+        call (a decoded token, or a further piece of a prompt that arrives in pieces).  Blocks of such sequences
+        are private (no forks, no content addressing)."""
+        assert not self.enable_caching and self.block_sliding_window is None
+        table = self.block_tables.setdefault(seq.seq_id, [])
+        while len(table) < seq.num_logical_blocks:
+            table.append(self.gpu_allocator.allocate())
+
     def fork(self, parent_seq: Sequence, child_seq: Sequence) -> None:
         src = self.block_tables[parent_seq.seq_id]
         self.block_tables[child_seq.seq_id] = list(src)

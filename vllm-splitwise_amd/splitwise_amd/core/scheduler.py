@@ -101,6 +101,13 @@ class Scheduler:
         # step has resolved, because the prompt GPU writes and pushes KV on its own clock
         self.in_flight: Callable[[Sequence], bool] = lambda seq: False
         self.held_after_abort: List[Sequence] = []
+        # ragged steps: every live sequence owns a slot of the workers' recurrent-state pools from its first
+        # portion to its release (a freed slot is the next one handed out, so slots are reused at once)
+        self.ragged_steps = bool(getattr(scheduler_config, "ragged_steps", False))
+        self.state_slots: Optional[SeqToSlotMapper] = (SeqToSlotMapper(scheduler_config.max_num_seqs)
+                                                       if self.ragged_steps else None)
+        # per scheduled group of the last ragged step: (group, sequence, tokens run, sampled?)
+        self.last_ragged: List[tuple] = []
 
     # -------------------------------------------------------------- queue admin
     def add_seq_group(self, seq_group: SequenceGroup) -> None:
@@ -300,6 +307,139 @@ class Scheduler:
         return SchedulerOutputs(self.running, False, num_batched_tokens, blocks_to_swap_in, blocks_to_swap_out,
                                 blocks_to_copy, coalesce_blocks_by_id(blocks_to_nw), [])
 
+    # ------------------------------------------------------------ ragged steps
+    def _ragged_admit(self, group: SequenceGroup, strict: bool) -> bool:
+        """Blocks for the tokens the waiting sequence has now and a state slot.  ``strict``: the caller has
+        decided that the group runs in this step (a replayed plan): no watermark is kept back."""
+        seq = group.get_seqs(status=SequenceStatus.WAITING)[0]
+        if self.state_slots.num_free() < 1:
+            return False
+        need = self.block_manager.blocks_missing(seq)
+        free = self.block_manager.get_num_free_gpu_blocks()
+        if need > (free if strict else free - self.block_manager.watermark_blocks):
+            return False
+        self.block_manager.extend(seq)
+        self.state_slots.set_seq(seq.seq_id)
+        seq.status = SequenceStatus.RUNNING
+        seq.num_computed_tokens = 0
+        return True
+
+    def _ragged_release(self, seq: Sequence) -> None:
+        self.block_manager.free(seq)
+        if seq.seq_id in self.state_slots:
+            self.state_slots.free_seq(seq.seq_id)
+
+    def _ragged_preempt(self, group: SequenceGroup) -> None:
+        """A recurrent state cannot be swapped out block by block: the sequence gives everything back and
+        is run again from its first token later."""
+        self.num_preemptions = getattr(self, "num_preemptions", 0) + 1
+        for seq in group.get_seqs(status=SequenceStatus.RUNNING):
+            seq.status = SequenceStatus.WAITING
+            seq.num_computed_tokens = 0
+            self._ragged_release(seq)
+        self.waiting.appendleft(group)
+
+    def schedule_ragged(self, plan: Optional[Dict[str, int]] = None,
+                        logits_at: Optional[Dict[str, List[int]]] = None
+                        ) -> Tuple[List[SequenceGroupMetadata], SchedulerOutputs]:
+        """One step that mixes portions of prompts with decoded tokens.
+
+        Without ``plan`` the step is filled by policy: every running sequence first (a decoded token, or the next
+        portion of its prompt), oldest first, then waiting prompts while blocks, state slots, the sequence
+        budget and the token budget allow; a prompt longer than what is left of the budget runs in portions.
+        With ``plan`` ({request id: tokens to run}) exactly those sequences run exactly that many of their next
+        tokens, nothing is sampled, and ``logits_at`` names the places whose logits are wanted: a recorded
+        schedule is replayed through the same admission, block and slot bookkeeping."""
+        assert self.ragged_steps
+        now = time.monotonic()
+        cfg = self.scheduler_config
+        chosen: List[tuple] = []                     # (group, sequence, tokens)
+        ignored: List[SequenceGroup] = []
+        if plan is not None:
+            by_id = {g.request_id: g for g in list(self.running) + list(self.waiting)}
+            for request_id, n in plan.items():
+                group = by_id.get(request_id)
+                if group is None:
+                    raise KeyError(f"request {request_id} is not live")
+                if group in self.waiting:
+                    if not self._ragged_admit(group, strict=True):
+                        raise RuntimeError(f"no blocks or no state slot left for request {request_id}")
+                    self.waiting.remove(group)
+                    self.running.append(group)
+                seq = group.get_seqs(status=SequenceStatus.RUNNING)[0]
+                if n < 1 or seq.num_computed_tokens + n > seq.get_len():
+                    raise ValueError(f"request {request_id}: {n} tokens asked, {seq.get_len() - seq.num_computed_tokens} left")
+                if self.block_manager.blocks_missing(seq) > self.block_manager.get_num_free_gpu_blocks():
+                    raise RuntimeError(f"no blocks left for request {request_id}")
+                self.block_manager.extend(seq)
+                chosen.append((group, seq, n))
+        else:
+            budget = cfg.max_num_batched_tokens
+            self.running = _fcfs_order(now, self.running)
+            kept: Deque[SequenceGroup] = deque()
+            while self.running:
+                group = self.running.popleft()
+                seq = group.get_seqs(status=SequenceStatus.RUNNING)[0]
+                ok = True
+                while self.block_manager.blocks_missing(seq) > self.block_manager.get_num_free_gpu_blocks():
+                    if self.running:
+                        self._ragged_preempt(self.running.pop())          # the youngest gives way
+                    else:
+                        self._ragged_preempt(group)
+                        ok = False
+                        break
+                if not ok:
+                    continue
+                kept.append(group)
+                left = seq.get_len() - seq.num_computed_tokens
+                if budget > 0 and left > 0:
+                    self.block_manager.extend(seq)
+                    n = min(left, budget)
+                    budget -= n
+                    chosen.append((group, seq, n))
+            self.running = kept
+            while self.waiting and budget > 0 and len(self.running) < cfg.max_num_seqs:
+                group = self.waiting[0]
+                seq = group.get_seqs(status=SequenceStatus.WAITING)[0]
+                if seq.get_len() > cfg.max_model_len or \
+                        seq.num_logical_blocks > self.block_manager.num_total_gpu_blocks - self.block_manager.watermark_blocks:
+                    seq.status = SequenceStatus.FINISHED_IGNORED
+                    ignored.append(group)
+                    self.waiting.popleft()
+                    continue
+                if not self._ragged_admit(group, strict=False):
+                    break
+                self.waiting.popleft()
+                self.running.append(group)
+                n = min(seq.get_len(), budget)
+                budget -= n
+                chosen.append((group, seq, n))
+        metas: List[SequenceGroupMetadata] = []
+        self.last_ragged = []
+        prompt_tokens = 0
+        for group, seq, n in chosen:
+            group.maybe_set_first_scheduled_time(now)
+            done = seq.num_computed_tokens
+            sample = plan is None and done + n == seq.get_len()
+            first_pass = done < seq.get_prompt_len()
+            prompt_tokens += n if first_pass else 0
+            metas.append(SequenceGroupMetadata(
+                request_id=group.request_id, is_prompt=first_pass, seq_data={seq.seq_id: seq.data},
+                sampling_params=group.sampling_params,
+                block_tables={seq.seq_id: self.block_manager.get_block_table(seq)}, computed_block_nums=[],
+                state=group.state, num_computed={seq.seq_id: done}, token_chunk={seq.seq_id: n},
+                state_slots={seq.seq_id: self.state_slots.get_slot_id(seq.seq_id)}, do_sample=sample,
+                logits_at=(logits_at or {}).get(group.request_id)))
+            self.last_ragged.append((group, seq, n, sample))
+        total = sum(n for _, _, n in chosen)
+        outputs = SchedulerOutputs([g for g, _, _ in chosen], prompt_tokens > 0, total, {}, {}, {}, {}, ignored)
+        # (SchedulerOutputs sorts by request id: metas follow the same order)
+        order = {g.request_id: i for i, g in enumerate(outputs.scheduled_seq_groups)}
+        metas.sort(key=lambda m: order[m.request_id])
+        self.last_ragged.sort(key=lambda e: order[e[0].request_id])
+        outputs.num_prompt_tokens = prompt_tokens
+        return metas, outputs
+
     def _metadata(self, outputs: SchedulerOutputs, groups: Iterable[SequenceGroup]) -> List[SequenceGroupMetadata]:
         now = time.monotonic()        # the clock of arrival_time: time_in_queue is a difference of the two
         metas: List[SequenceGroupMetadata] = []
@@ -323,6 +463,8 @@ class Scheduler:
         self.block_manager.mark_blocks_as_computed(seq_group)
 
     def schedule(self) -> Tuple[List[SequenceGroupMetadata], SchedulerOutputs]:
+        if self.ragged_steps:
+            return self.schedule_ragged()
         outputs = self._schedule()
         return self._metadata(outputs, outputs.scheduled_seq_groups), outputs
 
@@ -369,6 +511,8 @@ class Scheduler:
 
     def free_seq(self, seq: Sequence) -> None:
         self.block_manager.free(seq)
+        if self.state_slots is not None and seq.seq_id in self.state_slots:
+            self.state_slots.free_seq(seq.seq_id)
         if self.seq_to_slot_mapper is not None and seq.seq_id in self.seq_to_slot_mapper:
             self.seq_to_slot_mapper.free_seq(seq.seq_id)
         self._kv_pending.pop(seq.seq_id, None)

@@ -77,8 +77,16 @@ class EngineArgs:
             raise NotImplementedError("prefix caching needs the prompt pool to keep its blocks: it cannot be "
                                       "combined with staged_prompt_cache / token_pools > 1")
         model_config.verify_with_parallel_config(parallel_config)
-        scheduler_config = SchedulerConfig(self.max_num_batched_tokens, self.max_num_seqs,
+        ragged = model_config.uses_ragged_steps
+        if ragged and (self.pipeline_steps or self.sep_prompt_token or self.overlap_prompt_decode
+                       or self.enable_prefix_caching or self.tensor_parallel_size != 1):
+            raise NotImplementedError("models that run ragged steps (per-sequence recurrent state) run on one GPU, "
+                                      "step by step, without prefix caching")
+        max_tokens = self.max_num_batched_tokens
+        if ragged and max_tokens is None:
+            max_tokens = 2048                    # a prompt longer than the budget is run in portions
+        scheduler_config = SchedulerConfig(max_tokens, self.max_num_seqs,
                                            model_config.max_model_len, self.max_paddings,
                                            self.prefill_batch_tokens, self.prefill_max_wait,
-                                           self.pipeline_steps)
+                                           self.pipeline_steps, ragged_steps=ragged)
         return model_config, cache_config, parallel_config, scheduler_config, DeviceConfig(self.device)

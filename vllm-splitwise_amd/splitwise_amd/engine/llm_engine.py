@@ -71,6 +71,8 @@ class LLMEngine:
         self._staging_blocks = getattr(self.model_executor, "prompt_cache_blocks", None)
         if self.staged_prompt_cache and not self._staging_blocks:
             raise ValueError("staged_prompt_cache needs an executor that sizes the prompt pool's cache by itself")
+        self.ragged_steps = bool(getattr(scheduler_config, "ragged_steps", False))
+        self.last_logits: Dict[str, object] = {}
         self.stat_logger = None
         if log_stats:
             self.stat_logger = StatLogger(local_interval=5.0, labels=dict(model_name=model_config.model))
@@ -154,6 +156,9 @@ class LLMEngine:
             if self.tokenizer is None:
                 raise ValueError("prompt_token_ids must be given: no tokenizer is attached to this engine")
             prompt_token_ids = self.tokenizer.encode(prompt)
+        if sampling_params.best_of != 1 and self.ragged_steps:
+            raise NotImplementedError("n > 1 / best_of > 1 would have to copy a recurrent state per fork; "
+                                      "send n requests instead")
         if sampling_params.best_of != 1:
             # several sequences forked from one prompt (llm_engine.py:424-534).  Their blocks are shared copy-on-write
             # inside ONE cache; split pools would have to hand every fork's slot over, which the reference's
@@ -547,9 +552,77 @@ class LLMEngine:
         outputs += [RequestOutput.from_seq_group(g) for g in scheduler_outputs.ignored_seq_groups]
         return outputs
 
+    # ------------------------------------------------------------- ragged steps
+    def extend_request(self, request_id: str, token_ids: List[int]) -> None:
+        """Appends further tokens to a live request whose prompt arrives in pieces (nothing has been sampled
+        for it yet); the next steps run them."""
+        for queue in (self.scheduler.running, self.scheduler.waiting):
+            for group in queue:
+                if group.request_id == request_id:
+                    seq = group.get_seqs()[0]
+                    if seq.get_output_len():
+                        raise ValueError(f"request {request_id} has sampled tokens: its prompt cannot grow any more")
+                    seq.data.prompt_token_ids.extend(token_ids)
+                    return
+        raise KeyError(f"request {request_id} is not live")
+
+    def _step_ragged(self, plan: Optional[Dict[str, int]] = None,
+                     logits_at: Optional[Dict[str, List[int]]] = None) -> List[RequestOutput]:
+        """One step of a model that takes ragged batches: portions of prompts beside decoded tokens.  A sequence
+        whose portion ends before its last known token only advances; the others get a sampled token.  With a
+        ``plan`` (see Scheduler.schedule_ragged) nothing is sampled and ``self.last_logits`` holds the logits
+        asked for: {request id: fp32 tensor [places, vocab]}."""
+        scheduler = self.schedulers[0]
+        metas, outs = scheduler.schedule_ragged(plan, logits_at)
+        self.last_scheduled_prompt_run = bool(outs.prompt_run) and not outs.is_empty()
+        self.last_logits = {}
+        entries = list(scheduler.last_ragged)
+        if metas:
+            output = self.model_executor.execute_model(metas, {}, {}, {}, {})
+        else:
+            output = SamplerOutput([])
+        now, wall = time.monotonic(), time.time()
+        if output.logits is not None:
+            row = 0
+            for meta in metas:
+                k = len(meta.logits_at or ())
+                if k:
+                    self.last_logits[meta.request_id] = output.logits[row:row + k]
+                    row += k
+        reported: List[SequenceGroup] = []
+        for (group, seq, n, sampled), out in zip(entries, output):
+            seq.num_computed_tokens += n
+            if not sampled:
+                continue
+            sample = out.samples[0]
+            seq.append_token_id(sample.output_token, sample.logprobs)
+            self._decode_sequence(seq, group.sampling_params)
+            self._check_stop(seq, group.sampling_params)
+            if seq.is_finished():
+                scheduler.free_seq(seq)
+            group.maybe_set_first_token_time(wall)
+            reported.append(group)
+        scheduler.free_finished_seq_groups()
+        request_outputs = [RequestOutput.from_seq_group(g) for g in reported]
+        request_outputs += [RequestOutput.from_seq_group(g) for g in outs.ignored_seq_groups]
+        if self.stat_logger is not None:
+            self.stat_logger.log(self._get_stats(outs, reported, now))
+        return request_outputs
+
+    def step_planned(self, plan: Dict[str, int], logits_at: Optional[Dict[str, List[int]]] = None
+                     ) -> Dict[str, object]:
+        """Replays one recorded step: request id -> how many of its next tokens run now.  Returns the logits
+        asked for, {request id: fp32 [places, vocab]} (on the device)."""
+        if not self.ragged_steps:
+            raise NotImplementedError("planned steps need a model that runs ragged steps")
+        self._step_ragged(plan, logits_at or {})
+        return self.last_logits
+
     def step(self) -> List[RequestOutput]:
         """One scheduling decision, one model step on the executor, outputs appended
         (vllm/engine/llm_engine.py:571-633)."""
+        if self.ragged_steps:
+            return self._step_ragged()
         if self.pipeline_split:
             return self._step_split_pipelined()
         if self.overlap_pools:

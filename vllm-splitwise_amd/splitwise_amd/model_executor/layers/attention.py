@@ -218,3 +218,46 @@ class Attention(nn.Module):
             output = PagedAttentionImpl.forward_decode(query, key_cache, value_cache, input_metadata,
                                                        self.num_kv_heads, self.scale, self.alibi_slopes)
         return output.view(out_shape[:-1] + (self.num_heads * self.head_size,))
+
+
+class WindowTalkingAttention(nn.Module):
+    """Softmax attention without rotation over a sliding window plus a number of kept first tokens, with
+    the heads' weights mixed after the softmax by a learned [heads, heads] matrix, and with the RMS norm of
+    queries and keys taken over the whole projection (all heads at once) before the split into heads.
+
+    Keys (after their norm) and values live in a paged cache of this layer's own geometry
+    ([pages, page, kv_heads * size], token-major inside a page); a layer built with ``shares_kv`` has no key /
+    value projections and reads the cache of the layer it names.  Every page of a sequence is kept: the mask,
+    not the allocator, implements the window, so kept first tokens need no special pages."""
+
+    def __init__(self, heads: int, kv_heads: int, dim: int, vdim: int, scale: float, window: int, keep_first: int,
+                 eps: float, shares_kv: bool = False) -> None:
+        super().__init__()
+        assert heads % kv_heads == 0
+        self.heads, self.kv_heads, self.dim, self.vdim = heads, kv_heads, dim, vdim
+        self.scale, self.window, self.keep_first, self.eps = float(scale), int(window), int(keep_first), eps
+        self.shares_kv = shares_kv
+        self.q_norm = nn.Parameter(torch.ones(heads * dim, dtype=torch.float32), requires_grad=False)
+        self.k_norm = None if shares_kv else nn.Parameter(torch.ones(kv_heads * dim, dtype=torch.float32),
+                                                          requires_grad=False)
+        self.talk = nn.Parameter(torch.eye(heads, dtype=torch.float32), requires_grad=False)
+
+    def cache_shapes(self, block_size: int):
+        """Per page: keys, values."""
+        return [(block_size, self.kv_heads * self.dim), (block_size, self.kv_heads * self.vdim)]
+
+    def forward(self, q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.Tensor], key_cache: torch.Tensor,
+                value_cache: torch.Tensor, md: InputMetadata) -> torch.Tensor:
+        """q, k, v: column ranges of one projection output [rows, *]; k, v None for a layer that shares them."""
+        rows = q.shape[0]
+        q32 = torch.empty(rows, self.heads * self.dim, dtype=torch.float32, device=q.device)
+        if self.shares_kv:
+            _C.mixer_ops.qk_norm_cache(q32, q, None, None, self.q_norm.data, None, self.eps, None, None, None)
+        else:
+            _C.mixer_ops.qk_norm_cache(q32, q, k, v, self.q_norm.data, self.k_norm.data, self.eps, key_cache,
+                                       value_cache, md.slot_mapping)
+        out = torch.empty(rows, self.heads * self.vdim, dtype=q.dtype, device=q.device)
+        _C.mixer_ops.window_attention(out, q32, key_cache, value_cache, self.talk.data, md.ragged, self.heads,
+                                      self.kv_heads, self.dim, self.vdim, self.scale, self.window, self.keep_first,
+                                      tiled=md.ragged.max_query_len > 1)
+        return out

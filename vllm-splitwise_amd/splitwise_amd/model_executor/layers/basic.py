@@ -100,3 +100,28 @@ class SiluAndMul(nn.Module):
         out = torch.empty(x.shape[:-1] + (d,), dtype=x.dtype, device=x.device)
         _C.ops.silu_and_mul(out, x)
         return out
+
+
+class ScalarRMSNorm(nn.Module):
+    """RMS norm with ONE gain for all coordinates, applied to a sublayer's OUTPUT and added to an fp32
+    residual stream: residual += y / sqrt(mean(y^2) + eps) * g.  The gain is kept in fp32."""
+
+    def __init__(self, eps: float = 1e-6) -> None:
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(1, dtype=torch.float32), requires_grad=False)
+        self.variance_epsilon = eps
+
+    def _forward(self, residual: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
+        y = y.float()
+        return residual + y * torch.rsqrt(y.pow(2).mean(-1, keepdim=True) + self.variance_epsilon) * self.weight
+
+    def add_to(self, residual: torch.Tensor, y: torch.Tensor, cast_out: Optional[torch.Tensor] = None) -> None:
+        """In place on ``residual``; ``cast_out`` receives the new residual in the activation dtype (the next
+        sublayer's input)."""
+        _C.mixer_ops.scalar_norm_add(residual, y, self.weight.data, self.variance_epsilon, cast_out)
+
+    def forward(self, x: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+        """The model's final norm: fp32 stream in, activations out."""
+        out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+        _C.mixer_ops.scalar_norm(out, x, self.weight.data, self.variance_epsilon)
+        return out

@@ -1,0 +1,63 @@
+"""Mixture-of-experts feed-forward layers.
+
+``TableRoutedExperts``: no learned router -- a table [vocab, top] names each token id's experts, every chosen
+expert weighs 1 / top.  An expert is down(gelu(up x)) with the exact (erf) gelu and no biases.  An optional
+shared expert of the same form runs for every token and is added after a per-token sigmoid gate.
+
+Rows are grouped by expert on the device (a stable sort of the (row, choice) pairs by expert id and a prefix
+sum of the counts), so each expert's rows are one contiguous run of a gathered matrix.
+"""
+from typing import Dict, Optional
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from ... import _C
+from .linear import MergedColumnParallelLinear, RowParallelLinear
+
+
+class TableRoutedExperts(nn.Module):
+    def __init__(self, width: int, vocab: int, num_experts: int, top: int, ff: int, shared_ff: Optional[int],
+                 dtype: torch.dtype, linear_method=None) -> None:
+        super().__init__()
+        self.width, self.num_experts, self.top, self.ff = width, num_experts, top, ff
+        self.table = nn.Parameter(torch.zeros(vocab, top, dtype=torch.int32), requires_grad=False)
+        self.up = nn.Parameter(torch.empty(num_experts, ff, width, dtype=dtype), requires_grad=False)
+        self.down = nn.Parameter(torch.empty(num_experts, width, ff, dtype=dtype), requires_grad=False)
+        self.shared_ff = shared_ff
+        if shared_ff:
+            # shared expert's up projection and its gate read the same input: one GEMM
+            self.shared_in = MergedColumnParallelLinear(width, [shared_ff, 1], False, dtype, linear_method)
+            self.shared_down = RowParallelLinear(shared_ff, width, False, dtype, linear_method)
+
+    def route(self, token_ids: torch.Tensor):
+        """-> (order [rows * top] int32: pair index row * top + choice, sorted by expert;
+               expert_start [experts + 1] int32)."""
+        experts = self.table.data.index_select(0, token_ids).view(-1)              # [rows * top]
+        order = torch.sort(experts, stable=True).indices.to(torch.int32)
+        counts = torch.bincount(experts, minlength=self.num_experts)
+        start = torch.zeros(self.num_experts + 1, dtype=torch.int32, device=token_ids.device)
+        start[1:] = torch.cumsum(counts, 0)
+        return order, start
+
+    def forward(self, h: torch.Tensor, token_ids: torch.Tensor) -> torch.Tensor:
+        """-> fp32 [rows, width]: the experts' sum is accumulated in fp32."""
+        rows = h.shape[0]
+        order, start = self.route(token_ids)
+        out = torch.zeros(rows, self.width, dtype=torch.float32, device=h.device)
+        _C.mixer_ops.expert_ffn(out, h, self.up.data, self.down.data, order, start, self.top, 1.0 / self.top)
+        if self.shared_ff:
+            both = self.shared_in(h)
+            hidden = F.gelu(both[:, :self.shared_ff])
+            shared = self.shared_down(hidden)
+            out.addcmul_(torch.sigmoid(both[:, self.shared_ff:].float()), shared.float())
+        return out
+
+    def load_named(self, w: Dict[str, torch.Tensor]) -> None:
+        self.table.data.copy_(w["table"].to(torch.int32))
+        self.up.data.copy_(torch.stack([w[f"e{e}.up"] for e in range(self.num_experts)]))
+        self.down.data.copy_(torch.stack([w[f"e{e}.down"] for e in range(self.num_experts)]))
+        if self.shared_ff:
+            self.shared_in.weight.data.copy_(torch.cat([w["shared.up"], w["shared.sg"]], 0))
+            self.shared_down.weight.data.copy_(w["shared.down"])

@@ -1,0 +1,121 @@
+"""Token mixers with a per-sequence recurrent state: delta-rule layers and the short causal convolution
+in front of them.
+
+A layer's state lives in the worker's state pools (``worker/cache_engine.py``), one slot per live sequence:
+``state_shapes()`` names what the layer needs per slot, ``forward`` receives the allocated tensors.  All of a
+layer's projections of the same input are one GEMM; everything that enters the recurrence besides the
+projections (decays, step sizes, gates, unit norms, the state itself) is fp32 inside the kernels.
+
+Delta rule, per head, S [key size, value size] (keys index rows):
+  ``ChannelDeltaMixer``   S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
+                          g = exp(-exp(A_log) softplus(low-rank(h) + dt_bias)) per head and key channel
+  ``GeneralDeltaMixer``   S <- diag(w) S - (a * u)(u^T S) + k v^T;  o = S^T r,  u = k / |k|
+                          w = exp(-e^(-1/2) sigmoid(low-rank-tanh(h) + w0)),  a = sigmoid(W_a h + b)
+"""
+from typing import Dict, List, Tuple
+
+import torch
+import torch.nn as nn
+
+from ... import _C
+from ..input_metadata import InputMetadata
+from .linear import ColumnParallelLinear, MergedColumnParallelLinear, RowParallelLinear
+
+
+def _f32_param(*shape: int) -> nn.Parameter:
+    return nn.Parameter(torch.zeros(*shape, dtype=torch.float32), requires_grad=False)
+
+
+class ChannelDeltaMixer(nn.Module):
+    def __init__(self, width: int, heads: int, kv_heads: int, dim: int, vdim: int, conv_taps: int, decay_rank: int,
+                 gate_rank: int, eps: float, dtype: torch.dtype, linear_method=None) -> None:
+        super().__init__()
+        assert heads % kv_heads == 0
+        self.heads, self.kv_heads, self.dim, self.vdim, self.taps, self.eps = heads, kv_heads, dim, vdim, conv_taps, eps
+        self.conv_channels = 2 * kv_heads * dim + heads * vdim          # q | k | v
+        # q | k | v | beta | decay (low rank, first factor) | gate (low rank, first factor)
+        self.in_sizes = [kv_heads * dim, kv_heads * dim, heads * vdim, heads, decay_rank, gate_rank]
+        self.in_proj = MergedColumnParallelLinear(width, self.in_sizes, False, dtype, linear_method)
+        self.decay_up = ColumnParallelLinear(decay_rank, heads * dim, False, dtype, linear_method)
+        self.gate_up = ColumnParallelLinear(gate_rank, heads * vdim, False, dtype, linear_method)
+        self.o_proj = RowParallelLinear(heads * vdim, width, False, dtype, linear_method)
+        self.conv_taps = _f32_param(self.conv_channels, conv_taps)
+        self.dt_bias = _f32_param(heads * dim)
+        self.a_log = _f32_param(heads)
+        self.out_norm = nn.Parameter(torch.ones(vdim, dtype=torch.float32), requires_grad=False)
+
+    def state_shapes(self) -> List[Tuple[int, ...]]:
+        """Per slot: the convolution's last inputs, the delta-rule state."""
+        return [(self.taps - 1, self.conv_channels), (self.heads, self.dim, self.vdim)]
+
+    def forward(self, h: torch.Tensor, state: List[torch.Tensor], md: InputMetadata) -> torch.Tensor:
+        conv_state, rule_state = state
+        batch = md.ragged
+        rows = h.shape[0]
+        proj = self.in_proj(h)
+        c = self.conv_channels
+        beta_pre = proj[:, c:c + self.heads]
+        lo = c + self.heads
+        decay_pre = self.decay_up(proj[:, lo:lo + self.in_sizes[4]])
+        gate_pre = self.gate_up(proj[:, lo + self.in_sizes[4]:])
+        qkv = torch.empty(rows, c, dtype=torch.float32, device=h.device)
+        _C.mixer_ops.short_conv(qkv, proj[:, :c], self.conv_taps.data, conv_state, batch)
+        o = torch.empty(rows, self.heads * self.vdim, dtype=torch.float32, device=h.device)
+        _C.mixer_ops.channel_delta(o, qkv, beta_pre, decay_pre, self.dt_bias.data, self.a_log.data, rule_state, batch,
+                                   self.heads, self.kv_heads, self.dim, self.vdim)
+        gated = torch.empty(rows, self.heads * self.vdim, dtype=h.dtype, device=h.device)
+        _C.mixer_ops.head_norm_gate(gated, o, gate_pre, self.out_norm.data, False, self.eps, self.heads, self.vdim)
+        return self.o_proj(gated)
+
+    def load_named(self, w: Dict[str, torch.Tensor]) -> None:
+        """``w``: the layer's checkpoint tensors by their short names (q, q.conv, k, ..., o)."""
+        dev = self.dt_bias.device
+        self.in_proj.weight.data.copy_(torch.cat([w["q"], w["k"], w["v"], w["b"], w["a1"], w["g1"]], 0))
+        self.decay_up.weight.data.copy_(w["a2"])
+        self.gate_up.weight.data.copy_(w["g2"])
+        self.o_proj.weight.data.copy_(w["o"])
+        self.conv_taps.data.copy_(torch.cat([w["q.conv"], w["k.conv"], w["v.conv"]], 0).float().to(dev))
+        self.dt_bias.data.copy_(w["dt_bias"].float())
+        self.a_log.data.copy_(w["A_log"].float())
+        self.out_norm.data.copy_(w["norm"].float())
+
+
+class GeneralDeltaMixer(nn.Module):
+    def __init__(self, width: int, heads: int, dim: int, decay_rank: int, eps: float, dtype: torch.dtype,
+                 linear_method=None) -> None:
+        super().__init__()
+        self.heads, self.dim, self.eps = heads, dim, eps
+        size = heads * dim
+        self.size = size
+        # r | k | v | gate | removal rate | decay (low rank, first factor)
+        self.in_sizes = [size, size, size, size, size, decay_rank]
+        self.in_proj = MergedColumnParallelLinear(width, self.in_sizes, False, dtype, linear_method)
+        self.decay_up = ColumnParallelLinear(decay_rank, size, False, dtype, linear_method)
+        self.o_proj = RowParallelLinear(size, width, False, dtype, linear_method)
+        self.w0 = _f32_param(size)
+        self.rate_bias = _f32_param(size)
+        self.out_norm = nn.Parameter(torch.ones(size, dtype=torch.float32), requires_grad=False)
+
+    def state_shapes(self) -> List[Tuple[int, ...]]:
+        return [(self.heads, self.dim, self.dim)]
+
+    def forward(self, h: torch.Tensor, state: List[torch.Tensor], md: InputMetadata) -> torch.Tensor:
+        batch = md.ragged
+        rows, n = h.shape[0], self.size
+        proj = self.in_proj(h)
+        decay_pre = self.decay_up(torch.tanh(proj[:, 5 * n:]))
+        o = torch.empty(rows, n, dtype=torch.float32, device=h.device)
+        _C.mixer_ops.general_delta(o, proj[:, :n], proj[:, n:2 * n], proj[:, 2 * n:3 * n], decay_pre, self.w0.data,
+                                   proj[:, 4 * n:5 * n], self.rate_bias.data, state[0], batch, self.heads, self.dim)
+        gated = torch.empty(rows, n, dtype=h.dtype, device=h.device)
+        _C.mixer_ops.head_norm_gate(gated, o, proj[:, 3 * n:4 * n], self.out_norm.data, True, self.eps, self.heads,
+                                    self.dim)
+        return self.o_proj(gated)
+
+    def load_named(self, w: Dict[str, torch.Tensor]) -> None:
+        self.in_proj.weight.data.copy_(torch.cat([w["r"], w["k"], w["v"], w["g"], w["a"], w["w1"]], 0))
+        self.decay_up.weight.data.copy_(w["w2"])
+        self.o_proj.weight.data.copy_(w["o"])
+        self.w0.data.copy_(w["w0"].float())
+        self.rate_bias.data.copy_(w["a.b"].float())
+        self.out_norm.data.copy_(w["norm"].float())

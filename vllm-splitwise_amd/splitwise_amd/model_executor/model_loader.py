@@ -14,9 +14,27 @@ import torch.nn as nn
 
 from ..config import ModelConfig
 from .models.llama import LlamaForCausalLM
+from .models.nepevik import NepevikForCausalLM
 from .models.opt import OPTForCausalLM
 
-_ARCH = {"llama": LlamaForCausalLM, "opt": OPTForCausalLM}
+_ARCH = {"llama": LlamaForCausalLM, "opt": OPTForCausalLM, "nepevik": NepevikForCausalLM}
+
+
+def architecture_class(name: str):
+    try:
+        return _ARCH[name]
+    except KeyError:
+        raise ValueError(f"Model architecture {name!r} is not supported; known: {sorted(_ARCH)}") from None
+
+
+def _safetensors_shapes(path: str) -> dict:
+    """name -> shape from a safetensors header (8-byte length, then JSON), without reading the data."""
+    import json
+    import struct
+    with open(path, "rb") as f:
+        (n,) = struct.unpack("<Q", f.read(8))
+        header = json.loads(f.read(n))
+    return {k: tuple(v["shape"]) for k, v in header.items() if k != "__metadata__"}
 
 
 def _linear_method(model_config: ModelConfig):
@@ -76,7 +94,14 @@ def _random_init(model: nn.Module, seed: int) -> None:
 
 
 def get_model(model_config: ModelConfig, device: torch.device) -> nn.Module:
-    cls = _ARCH[model_config.architecture]
+    cls = architecture_class(model_config.architecture)
+    files = sorted(glob.glob(os.path.join(model_config.model, "*.safetensors"))) if os.path.isdir(
+        model_config.model) else []
+    if files and hasattr(cls, "note_tensor_shapes"):
+        shapes = {}
+        for f in files:
+            shapes.update(_safetensors_shapes(f))
+        cls.note_tensor_shapes(model_config.hf_config, shapes)
     # parameters created without an explicit dtype (norm weights) take the model dtype
     # (vllm/model_executor/model_loader.py:24-31 sets the default dtype the same way)
     old_dtype = torch.get_default_dtype()
@@ -86,16 +111,20 @@ def get_model(model_config: ModelConfig, device: torch.device) -> nn.Module:
             model = cls(model_config.hf_config, model_config.dtype, _linear_method(model_config))
     finally:
         torch.set_default_dtype(old_dtype)
-    files = sorted(glob.glob(os.path.join(model_config.model, "*.safetensors"))) if os.path.isdir(
-        model_config.model) else []
     if files:
         from safetensors.torch import load_file
         state = {}
         for f in files:
             state.update(load_file(f, device=str(device)))
-        missing, unexpected = model.load_state_dict(state, strict=False)
-        if missing:
-            raise ValueError(f"checkpoint {model_config.model} lacks parameters: {missing[:8]} ...")
+        if hasattr(model, "load_weights"):
+            with torch.no_grad():
+                model.load_weights(state)            # the model maps checkpoint names onto its (fused) parameters
+        else:
+            missing, unexpected = model.load_state_dict(state, strict=False)
+            if missing:
+                raise ValueError(f"checkpoint {model_config.model} lacks parameters: {missing[:8]} ...")
     else:
         _random_init(model, model_config.seed)
+        if hasattr(model, "finish_random_init"):
+            model.finish_random_init(model_config.seed)
     return model.eval()

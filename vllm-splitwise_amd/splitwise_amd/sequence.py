@@ -99,6 +99,8 @@ class Sequence:
         self.output_logprobs: List[Dict[int, Logprob]] = []
         self.output_text = ""
         self.status = SequenceStatus.WAITING
+        # ragged steps: tokens whose layers have run (their keys are cached, the recurrent state is past them)
+        self.num_computed_tokens = 0
         # incremental detokenisation state (engine-owned)
         self.prefix_offset = 0
         self.read_offset = 0
@@ -283,7 +285,19 @@ class SequenceGroupMetadata:
     def __init__(self, request_id: str, is_prompt: bool, seq_data: Dict[int, SequenceData],
                  sampling_params: SamplingParams, block_tables: Optional[Dict[int, List[int]]],
                  computed_block_nums: Optional[List[int]] = None,
-                 state: Optional[SequenceGroupState] = None) -> None:
+                 state: Optional[SequenceGroupState] = None,
+                 num_computed: Optional[Dict[int, int]] = None, token_chunk: Optional[Dict[int, int]] = None,
+                 state_slots: Optional[Dict[int, int]] = None, do_sample: bool = True,
+                 logits_at: Optional[List[int]] = None) -> None:
+        """Ragged steps add, per sequence id: ``num_computed`` (tokens earlier steps have run), ``token_chunk``
+        (how many of the following tokens this step runs), ``state_slots`` (its slot in the recurrent-state
+        pools); ``do_sample``: the step reaches the sequence's last known token and a new one is to be drawn;
+        ``logits_at``: places among this step's tokens whose logits the caller wants back."""
+        self.num_computed = num_computed
+        self.token_chunk = token_chunk
+        self.state_slots = state_slots
+        self.do_sample = do_sample
+        self.logits_at = logits_at
         self.request_id = request_id
         self.is_prompt = is_prompt
         self.seq_data = seq_data
@@ -329,6 +343,8 @@ class SamplerOutput:
     sampled_token_probs: Optional[object] = None
     sampled_token_ids: Optional[object] = None
     spec_decode_worker_metrics: Optional[object] = None
+    # fp32 [asked rows, vocab]: the logits that the step's commands asked for (``logits_at``), in command order
+    logits: Optional[object] = None
 
     def __getitem__(self, idx: int) -> SequenceGroupOutput:
         return self.outputs[idx]

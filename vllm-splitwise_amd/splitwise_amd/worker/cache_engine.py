@@ -120,3 +120,76 @@ class CacheEngine:
         per_tensor = block_size * num_heads * head_size
         dtype = _cache_torch_dtype(cache_dtype, model_config.dtype)
         return torch.tensor([], dtype=dtype).element_size() * num_layers * 2 * per_tensor
+
+
+class LayeredCacheEngine:
+    """Caches of a model whose layers differ (``ModelConfig.get_cache_layout``): per layer either pages of its
+    own shapes (the model's dtype), per-sequence state slots (fp32), or the tensors of an earlier layer.
+
+    ``gpu_cache[i]`` is the list of tensors that layer i's mixer receives: paged tensors are
+    [num_blocks, *shape per page], state tensors [num_slots, *shape per slot].  Pages are handed out by the
+    block manager, slots by the scheduler; a sequence that starts in a slot (or a page) ignores what an
+    earlier owner left there, so nothing is cleared on reuse.  Recurrent states cannot be swapped to the host
+    block by block: preemption recomputes (the scheduler's ragged mode never asks for a swap or a copy)."""
+
+    def __init__(self, cache_config: CacheConfig, model_config: ModelConfig, parallel_config: ParallelConfig,
+                 device: torch.device, num_state_slots: int) -> None:
+        self.cache_config = cache_config
+        self.block_size = cache_config.block_size
+        self.num_gpu_blocks = cache_config.num_gpu_blocks
+        self.num_cpu_blocks = 0
+        self.num_state_slots = num_state_slots
+        self.dtype = model_config.dtype
+        self.device = device
+        if cache_config.cache_dtype != "auto":
+            raise NotImplementedError("layered caches are kept in the model's dtype")
+        self.layout = model_config.get_cache_layout(self.block_size)
+        self.num_layers = len(self.layout)
+        self.gpu_cache = self.allocate(self.layout, self.num_gpu_blocks, num_state_slots, self.dtype, device)
+        self.events = []
+
+    @staticmethod
+    def allocate(layout, num_blocks: int, num_slots: int, dtype: torch.dtype, device: torch.device):
+        cache = []
+        for spec in layout:
+            if "alias" in spec:
+                cache.append(cache[spec["alias"]])
+            elif "paged" in spec:
+                cache.append([torch.zeros((num_blocks, *shape), dtype=dtype, device=device) for shape in spec["paged"]])
+            else:
+                cache.append([torch.zeros((num_slots, *shape), dtype=torch.float32, device=device)
+                              for shape in spec["state"]])
+        return cache
+
+    def swap_in(self, src_to_dst) -> None:
+        raise NotImplementedError("layered caches are not swapped: preemption recomputes")
+
+    swap_out = swap_in
+
+    def copy(self, src_to_dsts) -> None:
+        raise NotImplementedError("layered caches have no copy-on-write blocks")
+
+    @staticmethod
+    def get_cache_block_size(block_size: int, cache_dtype: str, model_config: ModelConfig,
+                             parallel_config: ParallelConfig) -> int:
+        """Bytes of one block over all layers that own pages."""
+        es = torch.tensor([], dtype=model_config.dtype).element_size()
+        total = 0
+        for spec in model_config.get_cache_layout(block_size):
+            for shape in spec.get("paged", ()):
+                n = 1
+                for d in shape:
+                    n *= d
+                total += n * es
+        return max(total, 1)
+
+    @staticmethod
+    def get_state_bytes(block_size: int, model_config: ModelConfig, num_slots: int) -> int:
+        total = 0
+        for spec in model_config.get_cache_layout(block_size):
+            for shape in spec.get("state", ()):
+                n = 4
+                for d in shape:
+                    n *= d
+                total += n * num_slots
+        return total

@@ -24,7 +24,7 @@ import numpy as np
 import torch
 
 from ..config import DeviceConfig, ModelConfig, ParallelConfig, SchedulerConfig
-from ..model_executor.input_metadata import InputMetadata
+from ..model_executor.input_metadata import InputMetadata, RaggedBatch
 from ..model_executor.layers.sampler import FollowerSamples, PendingSamples, SamplingMetadata
 from ..model_executor.model_loader import get_model
 from ..sampling_params import SamplingParams
@@ -251,8 +251,73 @@ class ModelRunner:
             token_tensor = torch.where((src >= 0).view(-1, 1), on_device, token_tensor)
         return (token_tensor, self._to_device(np.asarray(positions, dtype=np.int64).reshape(-1, 1), torch.long), md)
 
+    # ------------------------------------------------------------ ragged steps
+    def _prepare_ragged(self, metas: List[SequenceGroupMetadata]):
+        """Every sequence brings ``token_chunk`` tokens from position ``num_computed`` on, back to back.
+        -> (input_tokens [T], input_positions [T], InputMetadata, last row of every sequence, rows whose logits
+        are asked for)."""
+        bs = self.block_size
+        tokens: List[int] = []
+        positions: List[int] = []
+        slots: List[int] = []
+        token_seq: List[int] = []
+        q_start, ctx, state_slot, tables, last_rows, logit_rows = [0], [], [], [], [], []
+        for meta in metas:
+            (seq_id, data), = meta.seq_data.items()
+            done, n = meta.num_computed[seq_id], meta.token_chunk[seq_id]
+            ids = data.get_token_ids()
+            assert 0 < n and done + n <= len(ids), (done, n, len(ids))
+            table = meta.block_tables[seq_id]
+            assert len(table) * bs >= done + n, "the sequence's blocks do not cover this step's tokens"
+            first = len(tokens)
+            tokens += ids[done:done + n]
+            positions += range(done, done + n)
+            slots += [table[p // bs] * bs + p % bs for p in range(done, done + n)]
+            token_seq += [len(ctx)] * n
+            ctx.append(done)
+            state_slot.append(meta.state_slots[seq_id])
+            tables.append(table)
+            q_start.append(first + n)
+            last_rows.append(first + n - 1)
+            for place in meta.logits_at or ():
+                assert 0 <= place < n, (place, n)
+                logit_rows.append(first + place)
+        width = max(len(t) for t in tables)
+        i32 = lambda values: self._to_device(np.asarray(values, dtype=np.int32), torch.int32)   # noqa: E731
+        ragged = RaggedBatch(
+            q_start=i32(q_start), ctx_len=i32(ctx), token_seq=i32(token_seq), state_slot=i32(state_slot),
+            block_tables=self._to_device(_pad_2d(tables, width, 0, np.int32), torch.int32), num_seqs=len(ctx),
+            max_query_len=max(b - a for a, b in zip(q_start, q_start[1:])),
+            max_pages_used=max(-(-(c + b - a) // bs) for c, a, b in zip(ctx, q_start, q_start[1:])),
+            max_page_id=max(max(t) for t in tables), max_state_slot=max(state_slot))
+        md = InputMetadata(
+            is_prompt=ragged.max_query_len > 1, slot_mapping=self._to_device(np.asarray(slots, dtype=np.int64), torch.long),
+            prompt_lens=None, max_seq_len=None, start_loc=None, max_context_len=None, context_lens=None,
+            block_tables=None, use_cuda_graph=False, kv_cache_dtype=self.kv_cache_dtype, ragged=ragged)
+        return (self._to_device(np.asarray(tokens, dtype=np.int64), torch.long),
+                self._to_device(np.asarray(positions, dtype=np.int64), torch.long), md, last_rows, logit_rows)
+
+    @torch.inference_mode()
+    def _execute_ragged(self, metas: List[SequenceGroupMetadata], kv_caches) -> SamplerOutput:
+        from ..sequence import SequenceGroupOutput
+        tokens, positions, md, last_rows, logit_rows = self._prepare_ragged(metas)
+        hidden = self.model(tokens, positions, kv_caches, md)
+        sampling = [(meta, row) for meta, row in zip(metas, last_rows) if meta.do_sample]
+        sampled = {}
+        if sampling:
+            sampling_md = self._prepare_sample([m for m, _ in sampling], [r for _, r in sampling], as_prompts=True)
+            result = self.model.sample(hidden, sampling_md)
+            sampled = {m.request_id: out for (m, _), out in zip(sampling, result)}
+        output = SamplerOutput([sampled.get(m.request_id, SequenceGroupOutput([], None)) for m in metas])
+        if logit_rows:
+            rows = self._to_device(np.asarray(logit_rows, dtype=np.int64), torch.long)
+            output.logits = self.model.compute_logits(hidden.index_select(0, rows))
+        self.pending = None
+        return output
+
     # ---------------------------------------------------------------- sampling
-    def _prepare_sample(self, metas: List[SequenceGroupMetadata], last_token_rows: Optional[List[int]]):
+    def _prepare_sample(self, metas: List[SequenceGroupMetadata], last_token_rows: Optional[List[int]],
+                        as_prompts: bool = False):
         """Rows of the hidden states to sample from: the last token of every prompt, or every row
         of a decode step (model_runner.py:401-485 without prompt_logprobs)."""
         seq_groups: List[Tuple[List[int], SamplingParams]] = []
@@ -265,7 +330,7 @@ class ModelRunner:
             params = meta.sampling_params
             seq_groups.append((seq_ids, params))
             seq_data.update(meta.seq_data)
-            if meta.is_prompt:
+            if meta.is_prompt or as_prompts:          # one row per group, named by the caller
                 selected.append(last_token_rows[i])
                 n_rows = 1
             else:
@@ -300,6 +365,10 @@ class ModelRunner:
         which must all make this call the same way -- off for a prompt pool, whose ranks never decode.
         ``track_pending`` off: the step's samples are not what the next decode step continues from (a prompt step
         that runs beside the decode steps, on a stream of its own)."""
+        if metas[0].token_chunk is not None:
+            if defer:
+                raise NotImplementedError("ragged steps return their samples at once")
+            return self._execute_ragged(metas, kv_caches)
         is_prompt = metas[0].is_prompt
         restore = None
         if is_prompt:
@@ -396,6 +465,9 @@ class ModelRunner:
         params = SamplingParams(temperature=0.0, max_tokens=1)
         max_tokens = self.scheduler_config.max_num_batched_tokens
         max_seqs = self.scheduler_config.max_num_seqs
+        if self.model_config.uses_ragged_steps:
+            self._profile_ragged(params, max_tokens, max_seqs)
+            return
         metas = []
         for gid in range(max_seqs):
             n = max_tokens // max_seqs + (gid < max_tokens % max_seqs)
@@ -404,6 +476,27 @@ class ModelRunner:
             metas.append(SequenceGroupMetadata(str(gid), True, {gid: SequenceData([0] * n)}, params, None))
         num_layers = self.model_config.get_num_layers(self.parallel_config)
         self.execute_model(metas, [(None, None)] * num_layers)
+        if self.device.type == "cuda":
+            torch.cuda.synchronize()
+
+    def _profile_ragged(self, params: SamplingParams, max_tokens: int, max_seqs: int) -> None:
+        """The largest admissible step of a ragged model, against caches just big enough for it (they are part
+        of the measured peak, which errs on the safe side)."""
+        from .cache_engine import LayeredCacheEngine
+        bs = self.block_size or 16
+        self.block_size = bs
+        layout = self.model_config.get_cache_layout(bs)
+        metas, next_block = [], 0
+        for gid in range(max_seqs):
+            n = max_tokens // max_seqs + (gid < max_tokens % max_seqs)
+            if n == 0:
+                continue
+            blocks = list(range(next_block, next_block + -(-n // bs)))
+            next_block += len(blocks)
+            metas.append(SequenceGroupMetadata(str(gid), True, {gid: SequenceData([0] * n)}, params, {gid: blocks},
+                                               num_computed={gid: 0}, token_chunk={gid: n}, state_slots={gid: gid}))
+        caches = LayeredCacheEngine.allocate(layout, next_block, max_seqs, self.model_config.dtype, self.device)
+        self.execute_model(metas, caches)
         if self.device.type == "cuda":
             torch.cuda.synchronize()
 

@@ -19,7 +19,7 @@ import torch.distributed as dist
 from ..config import CacheConfig, DeviceConfig, ModelConfig, ParallelConfig, SchedulerConfig
 from ..model_executor import parallel_state
 from ..sequence import SamplerOutput, SequenceGroupMetadata
-from .cache_engine import CacheEngine
+from .cache_engine import CacheEngine, LayeredCacheEngine
 from .model_runner import ModelRunner
 
 
@@ -136,6 +136,10 @@ class Worker:
         free_gpu_memory, total_gpu_memory = torch.cuda.mem_get_info()
         peak_memory = self.init_gpu_memory - free_gpu_memory
         cache_block_size = self.get_cache_block_size_bytes(block_size, cache_dtype)
+        if self.model_config.get_cache_layout(block_size) is not None:
+            # the state slots are a fixed cost beside the pages
+            peak_memory += LayeredCacheEngine.get_state_bytes(block_size, self.model_config,
+                                                              self.scheduler_config.max_num_seqs)
         num_gpu_blocks = int((total_gpu_memory * gpu_memory_utilization - peak_memory) // cache_block_size)
         num_cpu_blocks = int(cpu_swap_space // cache_block_size)
         gc.collect()
@@ -144,13 +148,18 @@ class Worker:
 
     def init_cache_engine(self, cache_config: CacheConfig) -> None:
         self.cache_config = cache_config
-        self.cache_engine = CacheEngine(cache_config, self.model_config, self.parallel_config, self.device)
+        if self.model_config.get_cache_layout(cache_config.block_size) is not None:
+            self.cache_engine = LayeredCacheEngine(cache_config, self.model_config, self.parallel_config, self.device,
+                                                   num_state_slots=self.scheduler_config.max_num_seqs)
+        else:
+            self.cache_engine = CacheEngine(cache_config, self.model_config, self.parallel_config, self.device)
         self.gpu_cache = self.cache_engine.gpu_cache
         self.model_runner.set_block_size(self.cache_engine.block_size)
 
     def warm_up_model(self) -> None:
         # decode graphs; a prompt-pool worker never decodes
-        if not self.model_config.enforce_eager and not self.is_prompt_worker():
+        if (not self.model_config.enforce_eager and not self.is_prompt_worker()
+                and not self.model_config.uses_ragged_steps):       # ragged steps run eagerly
             self.model_runner.capture_model(self.gpu_cache)
         torch.manual_seed(self.model_config.seed)
 
@@ -346,4 +355,7 @@ class Worker:
         return {"total_ms": total_ms, "launches": launches, "alg_bytes": alg_bytes}
 
     def get_cache_block_size_bytes(self, block_size: int, cache_dtype: str) -> int:
+        if self.model_config.get_cache_layout(block_size) is not None:
+            return LayeredCacheEngine.get_cache_block_size(block_size, cache_dtype, self.model_config,
+                                                           self.parallel_config)
         return CacheEngine.get_cache_block_size(block_size, cache_dtype, self.model_config, self.parallel_config)
