@@ -111,6 +111,11 @@ def parse_args():
     ap.add_argument("--budget-s", type=float, default=840.0,
                     help="N > 1: legs after the headline leg are skipped once the run has taken this long")
     ap.add_argument("--leg-timeout", type=float, default=600.0, help="N > 1: longest any one leg may take (s)")
+    ap.add_argument("--mixers", action="store_true",
+                    help="instead of the headline workload: prefill / decode throughput of a Nepevik stack beside a Llama "
+                         "stack of equal size (random weights), and the mixer kernels beside the like Llama kernels with "
+                         "their distances from the roofline; one JSON line")
+    ap.add_argument("--mixer-sizes", default="2k", help="with --mixers: comma-separated preset sizes (2k, 4k)")
     ap.add_argument("--replica", default=None, help=argparse.SUPPRESS)          # set by the launcher
     ap.add_argument("--worker-cls", default=None, help=argparse.SUPPRESS)       # CPU dry runs of the launcher
     return ap.parse_args()
@@ -369,8 +374,18 @@ def cpu_baseline(model_name, prompt_len, decode_len):
             "sample": res["sample"]}
 
 
+def mixers_bench(args) -> None:
+    from splitwise_amd.executor import bench_mixers
+    result = bench_mixers.run(tuple(x for x in args.mixer_sizes.split(",") if x))
+    print(json.dumps({"metric": "nepevik_vs_llama_throughput", "unit": "tok/s", "n_gpus": 1, "dtype": "bf16",
+                      "data": "synthetic", **result}))
+
+
 def main():
     args = parse_args()
+    if args.mixers:
+        mixers_bench(args)
+        return
     if args.replica is not None:                     # one replica of a multi-GPU leg, started by the launcher
         from splitwise_amd.executor import bench_replica
         return bench_replica.run(json.loads(args.replica))

@@ -84,11 +84,14 @@ int swm_short_conv_advance(float* state, const void* x, int64_t x_stride, const 
  * qkv fp32 [rows, 2 * kv_heads * dim + heads * vdim] (q | k | v after the short convolution);
  * beta_pre act_dtype [rows, heads] (row stride beta_stride); decay_pre act_dtype [rows, heads * dim];
  * dt_bias fp32 [heads * dim]; a_log fp32 [heads]; state fp32 [slots, heads, dim, vdim];
- * out fp32 [rows, heads * vdim]. */
+ * out fp32 [rows, heads * vdim].  `workspace`: swm_channel_delta_workspace_floats() floats for the operands that
+ * a prologue kernel, parallel over tokens, prepares for the recurrence. */
+int64_t swm_channel_delta_workspace_floats(int64_t rows, int heads, int dim);
 int swm_channel_delta(float* out, const float* qkv, const void* beta_pre, int64_t beta_stride,
                       const void* decay_pre, const float* dt_bias, const float* a_log, float* state,
-                      const int32_t* q_start, const int32_t* ctx_len, const int32_t* state_slot,
-                      int num_seqs, int heads, int kv_heads, int dim, int vdim, int act_dtype, void* stream);
+                      const int32_t* q_start, const int32_t* ctx_len, const int32_t* state_slot, int64_t rows,
+                      int num_seqs, int heads, int kv_heads, int dim, int vdim, float* workspace, int act_dtype,
+                      void* stream);
 
 /* Delta rule with a decay and a removal rate per head and key channel:
  *   S <- diag(w) S - (a * u) (u^T S) + k v^T   (both terms read the old S);  o = S^T r
@@ -99,8 +102,9 @@ int swm_channel_delta(float* out, const float* qkv, const void* beta_pre, int64_
 int swm_general_delta(float* out, const void* r, const void* k, const void* v, int64_t rkv_stride,
                       const void* decay_pre, int64_t decay_stride, const float* w0, const void* rate_pre,
                       int64_t rate_stride, const float* a_bias, float* state, const int32_t* q_start,
-                      const int32_t* ctx_len, const int32_t* state_slot, int num_seqs, int heads, int dim,
-                      int act_dtype, void* stream);
+                      const int32_t* ctx_len, const int32_t* state_slot, int64_t rows, int num_seqs, int heads,
+                      int dim, float* workspace, int act_dtype, void* stream);
+int64_t swm_general_delta_workspace_floats(int64_t rows, int heads, int dim);
 
 /* out[t, h, :] = act_dtype(o / sqrt(mean(o^2) + eps) * weight[h * weight_head_stride + :] * sigmoid(gate[t, h, :]))
  * o fp32 [rows, heads * vdim]; gate act_dtype (row stride gate_stride); weight fp32. */

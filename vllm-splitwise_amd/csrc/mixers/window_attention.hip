@@ -143,6 +143,202 @@ __global__ __launch_bounds__(kAttnThreads) void window_attention_token_kernel(
   }
 }
 
+// ------------------------------------------------------------------------------------------ staged kernel
+// One workgroup per new token, all heads together.  A tile of 16 keys and their values (every key/value head) is
+// staged ONCE in LDS as fp32 and shared by all heads: scores by threads (head, key), the running softmax by one
+// thread per head, the value accumulation by threads (head, 8 value channels) for all key/value heads.  Needs
+// key size % 4 == 0, value size % 8 == 0 and whole 16-byte vectors per cached row; other shapes take the
+// kernel above.
+constexpr int kTileKeys = 16;
+constexpr int kKeyPad = 4;           // floats between staged key rows: 16 keys fall on 16 different bank groups
+
+template <typename T>
+__device__ __forceinline__ void stage_rows(float* __restrict__ dst, int dst_stride, const void* __restrict__ cache,
+                                           const int64_t* __restrict__ phys, int row_elems) {
+  // kTileKeys rows of `row_elems` cache elements -> fp32; phys[k] < 0: a row of zeros
+  constexpr int V = sizeof(typename Conv<T>::store_t) == 2 ? 8 : 4;          // elements per 16-byte vector
+  const int per_row = row_elems / V;
+  for (int e = threadIdx.x; e < kTileKeys * per_row; e += kAttnThreads) {
+    const int k = e / per_row, off = (e % per_row) * V;
+    float* d = dst + k * dst_stride + off;
+    if (phys[k] < 0) {
+#pragma unroll
+      for (int i = 0; i < V; ++i) d[i] = 0.0f;
+      continue;
+    }
+    const uint4 raw = *reinterpret_cast<const uint4*>(static_cast<const char*>(cache) +
+                                                      (phys[k] * row_elems + off) * sizeof(typename Conv<T>::store_t));
+    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+    if (V == 8) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        d[2 * i] = __uint_as_float(w[i] << 16);
+        d[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) d[i] = __uint_as_float(w[i]);
+    }
+  }
+}
+
+// NR: (head, 8-channel chunk) items per thread; GMAX >= kv_heads
+template <typename T, int GMAX, int NR>
+__global__ __launch_bounds__(kAttnThreads) void window_attention_staged_kernel(
+    void* __restrict__ out, const float* __restrict__ q, const void* __restrict__ key_cache,
+    const void* __restrict__ value_cache, const float* __restrict__ talk, const int32_t* __restrict__ block_tables,
+    int table_width, const int32_t* __restrict__ q_start, const int32_t* __restrict__ ctx_len,
+    const int32_t* __restrict__ token_seq, int heads, int kv_heads, int dim, int vdim, int page_size, float scale,
+    int window, int keep_first) {
+  extern __shared__ float lds[];
+  const int krow = kv_heads * dim + kKeyPad, vrow = kv_heads * vdim;
+  float* q_lds = lds;                                   // [heads * dim]
+  float* p_lds = q_lds + heads * dim;                   // [heads][16] scores, then weights
+  float* corr_lds = p_lds + heads * kTileKeys;          // [heads]
+  float* inv_lds = corr_lds + heads;                    // [heads]
+  float* k_lds = inv_lds + heads + (2 * heads) % 4;     // [16][krow], on a 16-byte boundary (2 * heads is even)
+  float* v_lds = k_lds + kTileKeys * krow;              // [16][vrow]
+  __shared__ int64_t phys[kTileKeys];
+  float* mixed = k_lds;                                 // [heads][kv_heads][vdim] once the tiles are done
+  const int64_t t = blockIdx.x;
+  const int s = token_seq[t];
+  const int i = ctx_len[s] + (int)(t - q_start[s]);
+  for (int e = threadIdx.x; e < heads * dim; e += kAttnThreads) q_lds[e] = q[t * (int64_t)heads * dim + e];
+  const int32_t* table = block_tables + (int64_t)s * table_width;
+  const int lo = max(0, i - window + 1);
+  const int n_first = min(keep_first, lo);
+  const int total = n_first + (i - lo + 1);
+  const int group = heads / kv_heads;
+  const int chunks = vdim / 8;                          // per head
+  float acc[NR][GMAX][8];
+#pragma unroll
+  for (int r = 0; r < NR; ++r)
+#pragma unroll
+    for (int c = 0; c < GMAX; ++c)
+#pragma unroll
+      for (int x = 0; x < 8; ++x) acc[r][c][x] = 0.0f;
+  float m_run = -INFINITY, l_run = 0.0f;                // of head threadIdx.x (threads < heads)
+  for (int base = 0; base < total; base += kTileKeys) {
+    __syncthreads();                                    // the previous tile is consumed (and q_lds is written)
+    if (threadIdx.x < kTileKeys) {
+      const int idx = base + threadIdx.x;
+      int64_t ph = -1;
+      if (idx < total) {
+        const int j = idx < n_first ? idx : lo + idx - n_first;
+        ph = (int64_t)table[j / page_size] * page_size + j % page_size;
+      }
+      phys[threadIdx.x] = ph;
+    }
+    __syncthreads();
+    stage_rows<T>(k_lds, krow, key_cache, phys, kv_heads * dim);
+    stage_rows<T>(v_lds, vrow, value_cache, phys, vrow);
+    __syncthreads();
+    for (int item = threadIdx.x; item < heads * kTileKeys; item += kAttnThreads) {
+      const int g = item / kTileKeys, k = item % kTileKeys;
+      const float4* qv = reinterpret_cast<const float4*>(q_lds + g * dim);
+      const float4* kv = reinterpret_cast<const float4*>(k_lds + k * krow + (g / group) * dim);
+      float sc = 0.0f;
+      for (int d4 = 0; d4 < dim / 4; ++d4) {
+        const float4 a = qv[d4], b = kv[d4];
+        sc += a.x * b.x + a.y * b.y + a.z * b.z + a.w * b.w;
+      }
+      p_lds[item] = base + k < total ? sc * scale : -INFINITY;
+    }
+    __syncthreads();
+    if (threadIdx.x < heads) {
+      float* p = p_lds + threadIdx.x * kTileKeys;
+      float m_new = m_run;
+#pragma unroll
+      for (int k = 0; k < kTileKeys; ++k) m_new = fmaxf(m_new, p[k]);
+      const float corr = expf(m_run - m_new);           // 0 at the first tile
+      float sum = 0.0f;
+#pragma unroll
+      for (int k = 0; k < kTileKeys; ++k) {
+        const float w = expf(p[k] - m_new);             // 0 for keys past the end
+        p[k] = w;
+        sum += w;
+      }
+      l_run = l_run * corr + sum;
+      m_run = m_new;
+      corr_lds[threadIdx.x] = corr;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < NR; ++r) {
+      const int item = threadIdx.x + r * kAttnThreads;
+      if (item >= heads * chunks) continue;
+      const int g = item / chunks, ch = item % chunks;
+      const float corr = corr_lds[g];
+#pragma unroll
+      for (int c = 0; c < GMAX; ++c)
+#pragma unroll
+        for (int x = 0; x < 8; ++x) acc[r][c][x] *= corr;
+      const float* p = p_lds + g * kTileKeys;
+#pragma unroll 4
+      for (int k = 0; k < kTileKeys; ++k) {
+        const float w = p[k];
+#pragma unroll
+        for (int c = 0; c < GMAX; ++c) {
+          if (c < kv_heads) {
+            const float4* vv = reinterpret_cast<const float4*>(v_lds + k * vrow + c * vdim + ch * 8);
+            const float4 a = vv[0], b = vv[1];
+            acc[r][c][0] += w * a.x; acc[r][c][1] += w * a.y; acc[r][c][2] += w * a.z; acc[r][c][3] += w * a.w;
+            acc[r][c][4] += w * b.x; acc[r][c][5] += w * b.y; acc[r][c][6] += w * b.z; acc[r][c][7] += w * b.w;
+          }
+        }
+      }
+    }
+  }
+  if (threadIdx.x < heads) inv_lds[threadIdx.x] = 1.0f / l_run;
+  __syncthreads();                                      // tiles are done: their space becomes `mixed`
+#pragma unroll
+  for (int r = 0; r < NR; ++r) {
+    const int item = threadIdx.x + r * kAttnThreads;
+    if (item >= heads * chunks) continue;
+    const int g = item / chunks, ch = item % chunks;
+    const float inv = inv_lds[g];
+#pragma unroll
+    for (int c = 0; c < GMAX; ++c)
+      if (c < kv_heads)
+#pragma unroll
+        for (int x = 0; x < 8; ++x) mixed[((int64_t)g * kv_heads + c) * vdim + ch * 8 + x] = acc[r][c][x] * inv;
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < heads * vdim; e += kAttnThreads) {
+    const int h = e / vdim, d = e % vdim;
+    const int c = h / group;
+    float o = 0.0f;
+    for (int g = 0; g < heads; ++g) o += talk[h * heads + g] * mixed[((int64_t)g * kv_heads + c) * vdim + d];
+    st<T>(out, t * (int64_t)heads * vdim + e, o);
+  }
+}
+
+inline size_t staged_lds_bytes(int heads, int kv_heads, int dim, int vdim) {
+  const size_t tiles = (size_t)kTileKeys * (kv_heads * dim + kKeyPad) + (size_t)kTileKeys * kv_heads * vdim;
+  const size_t mixed = (size_t)heads * kv_heads * vdim;
+  // `mixed` lies over the tiles, which come last
+  const size_t body = (size_t)heads * dim + (tiles > mixed ? tiles : mixed) + (size_t)heads * (kTileKeys + 2) + 2;
+  return body * sizeof(float);
+}
+
+template <typename T, int GMAX, int NR>
+int launch_staged(void* out, const float* q, const void* key_cache, const void* value_cache, const float* talk,
+                  const int32_t* block_tables, int table_width, const int32_t* q_start, const int32_t* ctx_len,
+                  const int32_t* token_seq, int64_t rows, int heads, int kv_heads, int dim, int vdim, int page_size,
+                  float scale, int window, int keep_first, hipStream_t stream) {
+  const size_t lds = staged_lds_bytes(heads, kv_heads, dim, vdim);
+  auto kernel = window_attention_staged_kernel<T, GMAX, NR>;
+  if (lds > 64 * 1024) {
+    SW_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     (int)lds));
+  }
+  hipLaunchKernelGGL(kernel, dim3((unsigned)rows), dim3(kAttnThreads), lds, stream, out, q, key_cache, value_cache,
+                     talk, block_tables, table_width, q_start, ctx_len, token_seq, heads, kv_heads, dim, vdim,
+                     page_size, scale, window, keep_first);
+  SW_CHECK_LAUNCH();
+  return SW_OK;
+}
+
 template <typename T, int GMAX, int NV>
 int launch_token(void* out, const float* q, const void* key_cache, const void* value_cache, const float* talk,
                  const int32_t* block_tables, int table_width, const int32_t* q_start, const int32_t* ctx_len,
@@ -198,6 +394,19 @@ int swm_window_attention(void* out, const float* q, const void* key_cache, const
   hipStream_t s = static_cast<hipStream_t>(stream);
   (void)tiled;
   (void)num_seqs;
+  // the staged kernel for shapes made of whole vectors whose accumulators fit the registers
+  const int vec = act_dtype == SW_BF16 ? 8 : 4;
+  const int items = heads * (vdim / 8);
+  const int nr = (items + kAttnThreads - 1) / kAttnThreads;
+  const int gmax = kv_heads <= 1 ? 1 : kv_heads <= 2 ? 2 : kv_heads <= 4 ? 4 : kv_heads <= 8 ? 8 : 16;
+  if (dim % 4 == 0 && vdim % 8 == 0 && (kv_heads * dim) % vec == 0 && (kv_heads * vdim) % vec == 0 && heads <= kAttnThreads &&
+      nr * gmax <= 16 && nr <= 4 && staged_lds_bytes(heads, kv_heads, dim, vdim) <= 150 * 1024) {
+    SWM_DISPATCH_ACT(act_dtype, SWM_DISPATCH_G(kv_heads, {
+      if (nr <= 1) return (launch_staged<T, GMAX, 1>(out, q, key_cache, value_cache, talk, block_tables, table_width, q_start, ctx_len, token_seq, rows, heads, kv_heads, dim, vdim, page_size, scale, window, keep_first, s));
+      if (nr <= 2) return (launch_staged<T, GMAX, 2>(out, q, key_cache, value_cache, talk, block_tables, table_width, q_start, ctx_len, token_seq, rows, heads, kv_heads, dim, vdim, page_size, scale, window, keep_first, s));
+      return (launch_staged<T, GMAX, 4>(out, q, key_cache, value_cache, talk, block_tables, table_width, q_start, ctx_len, token_seq, rows, heads, kv_heads, dim, vdim, page_size, scale, window, keep_first, s));
+    }););
+  }
   SWM_DISPATCH_ACT(act_dtype, SWM_DISPATCH_G(kv_heads, SWM_DISPATCH_NV(vdim, return (launch_token<T, GMAX, NV>(
       out, q, key_cache, value_cache, talk, block_tables, table_width, q_start, ctx_len, token_seq, rows, heads,
       kv_heads, dim, vdim, page_size, scale, window, keep_first, s)););););

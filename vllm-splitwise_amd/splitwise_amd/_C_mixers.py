@@ -32,8 +32,8 @@ _SIGNATURES = {
                              _i, _p],
     "swm_short_conv": [_p, _p, _l, _p, _p, _p, _p, _p, _p, _l, _i, _i, _i, _p],
     "swm_short_conv_advance": [_p, _p, _l, _p, _p, _p, _i, _i, _i, _i, _p],
-    "swm_channel_delta": [_p, _p, _p, _l, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p],
-    "swm_general_delta": [_p, _p, _p, _p, _l, _p, _l, _p, _p, _l, _p, _p, _p, _p, _p, _i, _i, _i, _i, _p],
+    "swm_channel_delta": [_p, _p, _p, _l, _p, _p, _p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p, _i, _p],
+    "swm_general_delta": [_p, _p, _p, _p, _l, _p, _l, _p, _p, _l, _p, _p, _p, _p, _p, _l, _i, _i, _i, _p, _i, _p],
     "swm_head_norm_gate": [_p, _p, _p, _l, _p, _i, _f, _l, _i, _i, _i, _p],
     "swm_expert_up_gelu": [_p, _p, _p, _p, _p, _i, _l, _i, _i, _i, _i, _p],
     "swm_expert_down": [_p, _p, _p, _p, _p, _i, _l, _i, _i, _i, _f, _i, _p],
@@ -248,8 +248,9 @@ def channel_delta(out: torch.Tensor, qkv: torch.Tensor, beta_pre: torch.Tensor, 
         _check(load_library().swm_channel_delta(
             out.data_ptr(), qkv.data_ptr(), beta_pre.data_ptr(), _rows(beta_pre, "beta_pre"), decay_pre.data_ptr(),
             dt_bias.data_ptr(), a_log.data_ptr(), state.data_ptr(), batch.q_start.data_ptr(),
-            batch.ctx_len.data_ptr(), batch.state_slot.data_ptr(), n, heads, kv_heads, dim, vdim, _act(decay_pre),
-            _stream(qkv)))
+            batch.ctx_len.data_ptr(), batch.state_slot.data_ptr(), rows, n, heads, kv_heads, dim, vdim,
+            torch.empty(rows * heads * (3 * dim + 1), dtype=torch.float32, device=qkv.device).data_ptr(),
+            _act(decay_pre), _stream(qkv)))
 
 
 def general_delta(out: torch.Tensor, r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay_pre: torch.Tensor,
@@ -271,7 +272,9 @@ def general_delta(out: torch.Tensor, r: torch.Tensor, k: torch.Tensor, v: torch.
             out.data_ptr(), r.data_ptr(), k.data_ptr(), v.data_ptr(), stride, decay_pre.data_ptr(),
             _rows(decay_pre, "decay_pre"), w0.data_ptr(), rate_pre.data_ptr(), _rows(rate_pre, "rate_pre"),
             a_bias.data_ptr(), state.data_ptr(), batch.q_start.data_ptr(), batch.ctx_len.data_ptr(),
-            batch.state_slot.data_ptr(), n, heads, dim, _act(r), _stream(r)))
+            batch.state_slot.data_ptr(), rows, n, heads, dim,
+            torch.empty(rows * heads * 4 * dim, dtype=torch.float32, device=r.device).data_ptr(), _act(r),
+            _stream(r)))
 
 
 def head_norm_gate(out: torch.Tensor, o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, per_head_weight: bool,

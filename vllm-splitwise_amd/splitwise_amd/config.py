@@ -37,6 +37,44 @@ MODEL_PRESETS = {
                      num_attention_heads=2, num_key_value_heads=2, intermediate_size=256,
                      max_position_embeddings=2048, torch_dtype="float16"),
 }
+
+
+def _nepevik_preset(width: int, repeats: int, heads: int, kv_heads: int, experts: int, top: int, ff: int) -> dict:
+    """A Nepevik stack of layer sizes that resemble a served model's: per repeat one windowed attention layer, two
+    channel-decay delta layers, one general delta layer and one attention layer that reads the first one's keys."""
+    d = width // heads
+    mlp = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top}, "shared": {"ff": 2 * ff}}
+    layers = []
+    for _ in range(repeats):
+        first = len(layers)
+        attn = {"heads": heads, "kv_heads": kv_heads, "dim": d, "vdim": d, "scale": d ** -0.5,
+                "mask": {"size": 1024, "keep_first": 16}}
+        delta = {"heads": heads, "kv_heads": heads, "dim": d, "vdim": d, "conv": 4}
+        layers += [{"type": "attention", "mixer": dict(attn), "mlp": mlp},
+                   {"type": "channel_delta", "mixer": dict(delta), "mlp": mlp},
+                   {"type": "channel_delta", "mixer": dict(delta), "mlp": mlp},
+                   {"type": "general_delta", "mixer": {"heads": 2 * heads, "dim": d // 2}, "mlp": mlp},
+                   {"type": "attention", "mixer": dict(attn, kv_from=first), "mlp": mlp}]
+    from .model_executor.models.nepevik import normalize_config
+    return normalize_config({"architecture": "Nepevik", "layers": layers, "norm": {"eps": 1e-6}, "vocab": 32000,
+                             "width": width})
+
+
+_NEPEVIK_PRESETS = {
+    # name: (width, repeats of the 5-layer pattern, heads, kv heads, experts, top, expert ff)
+    "nepevik-2k": (2048, 2, 16, 4, 32, 2, 1024),
+    "nepevik-4k": (4096, 2, 32, 8, 32, 2, 2048),
+}
+# Llama stacks of the same width, depth and active feed-forward size, to measure the above against
+MODEL_PRESETS.update({
+    "llama-2k": dict(architecture="llama", vocab_size=32000, hidden_size=2048, num_hidden_layers=10,
+                     num_attention_heads=16, num_key_value_heads=4, intermediate_size=2816,
+                     max_position_embeddings=8192, rms_norm_eps=1e-5, rope_theta=10000.0, torch_dtype="bfloat16"),
+    "llama-4k": dict(architecture="llama", vocab_size=32000, hidden_size=4096, num_hidden_layers=10,
+                     num_attention_heads=32, num_key_value_heads=8, intermediate_size=5632,
+                     max_position_embeddings=8192, rms_norm_eps=1e-5, rope_theta=10000.0, torch_dtype="bfloat16"),
+})
+
 _ALIASES = {
     "facebook/opt-125m": "opt-125m", "meta-llama/Llama-2-7b-hf": "llama-2-7b",
     "meta-llama/Llama-2-13b-hf": "llama-2-13b", "meta-llama/Llama-2-70b-hf": "llama-2-70b",
@@ -83,6 +121,8 @@ class ModelConfig:
         name = _ALIASES.get(model, model)
         if name in MODEL_PRESETS:
             return dict(MODEL_PRESETS[name])
+        if name in _NEPEVIK_PRESETS:
+            return _nepevik_preset(*_NEPEVIK_PRESETS[name])
         cfg_path = os.path.join(model, "config.json")
         if os.path.isfile(cfg_path):
             with open(cfg_path) as f:

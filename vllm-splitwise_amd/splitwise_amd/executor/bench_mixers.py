@@ -1,0 +1,258 @@
+"""Throughput of a Nepevik stack beside a Llama stack of the same width, depth and active feed-forward size
+(random weights), and every mixer kernel beside the like kernel of the Llama path with their distances from
+the roofline.  ``bench.py --mixers`` prints the result as one JSON line.
+
+Engine level: PREFILL = prompt tokens per second from the first step to the last prompt's first token;
+DECODE = generated tokens per second over a run of pure decode steps at a fixed batch.  Both go through
+``LLMEngine.step`` (scheduler, block tables, sampler), so host time counts.
+
+Kernel level: HIP-event time per launch; ``roof`` = the larger of (algorithmic bytes / HBM peak) and
+(flops / the unit's peak) divided by the measured time: 1.0 would be the roofline.  Matrix work on MFMA is
+priced at the dense bf16 peak, everything else at the fp32 vector peak.
+"""
+import time
+from typing import Dict, List
+
+import torch
+
+HBM_BPS = 8.0e12
+MFMA_BF16 = 2.5e15
+VALU_F32 = 157.0e12          # 256 CUs x 4 SIMDs x 16 lanes x 2 (fma) x 2 (dual issue not counted) x 2.4 GHz
+
+
+def _sync() -> None:
+    torch.cuda.synchronize()
+
+
+def engine_throughput(model: str, prompt_len: int = 2048, prompts: int = 8, decode_batch: int = 64,
+                      decode_prompt: int = 512, decode_steps: int = 48, budget: int = 4096) -> Dict[str, float]:
+    from ..engine.arg_utils import EngineArgs
+    from ..engine.llm_engine import LLMEngine
+    from ..sampling_params import SamplingParams
+    block = 16
+    need = max(prompts * (prompt_len + block), decode_batch * (decode_prompt + decode_steps + 2 * block))
+    engine = LLMEngine.from_engine_args(EngineArgs(
+        model=model, dtype="bfloat16", block_size=block, max_model_len=max(prompt_len, decode_prompt + decode_steps) + block,
+        max_num_seqs=max(decode_batch, prompts), max_num_batched_tokens=max(budget, prompt_len + block),
+        num_gpu_blocks_override=need // block + 64, swap_space=0))
+    vocab = engine.model_config.get_vocab_size()
+    gen = torch.Generator().manual_seed(0)
+
+    def tokens(n):
+        return torch.randint(0, vocab, (n,), generator=gen).tolist()
+
+    def drain():
+        while engine.has_unfinished_requests():
+            engine.step()
+
+    out = {}
+    for rep in range(2):                                   # the first pass warms libraries and allocators up
+        for i in range(prompts):
+            engine.add_request(f"p{rep}-{i}", None, SamplingParams(temperature=0.0, max_tokens=1, ignore_eos=True),
+                               prompt_token_ids=tokens(prompt_len))
+        _sync()
+        t0 = time.perf_counter()
+        drain()
+        _sync()
+        out["prefill_tok_s"] = prompts * prompt_len / (time.perf_counter() - t0)
+    for i in range(decode_batch):
+        engine.add_request(f"d{i}", None, SamplingParams(temperature=0.0, max_tokens=decode_steps + 8, ignore_eos=True),
+                           prompt_token_ids=tokens(decode_prompt))
+    # run until every request has its first token and a few decode steps have gone by
+    while any(len(g.get_seqs()[0].get_output_token_ids()) < 4 for g in engine.scheduler.running) or engine.scheduler.waiting:
+        engine.step()
+    _sync()
+    t0 = time.perf_counter()
+    for _ in range(decode_steps - 8):
+        engine.step()
+    _sync()
+    out["decode_tok_s"] = decode_batch * (decode_steps - 8) / (time.perf_counter() - t0)
+    out["decode_ms_per_step"] = 1e3 * decode_batch / out["decode_tok_s"]
+    drain()
+    del engine
+    torch.cuda.empty_cache()
+    return out
+
+
+def _time(fn, iters: int = 20, warmup: int = 3) -> float:
+    for _ in range(warmup):
+        fn()
+    _sync()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(iters):
+        fn()
+    b.record()
+    _sync()
+    return a.elapsed_time(b) / iters * 1e-3
+
+
+def _row(name: str, phase: str, t: float, nbytes: float, flops: float, peak: float, like: str = "") -> dict:
+    floor = max(nbytes / HBM_BPS, flops / peak)
+    return {"kernel": name, "phase": phase, "us": round(t * 1e6, 1), "GBps": round(nbytes / t / 1e9, 1),
+            "TFLOPs": round(flops / t / 1e12, 2), "roof": round(floor / t, 4), "like": like}
+
+
+def _ragged(seqs, dev):
+    """[(ctx, new tokens, slot, table)] -> an object with the ragged layout's tensors."""
+    from types import SimpleNamespace
+    q_start, token_seq = [0], []
+    for i, (_, n, _, _) in enumerate(seqs):
+        q_start.append(q_start[-1] + n)
+        token_seq += [i] * n
+    width = max(max(len(s[3]) for s in seqs), 1)
+    tables = torch.zeros(len(seqs), width, dtype=torch.int32)
+    for i, s in enumerate(seqs):
+        tables[i, :len(s[3])] = torch.tensor(s[3], dtype=torch.int32)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=dev)        # noqa: E731
+    return SimpleNamespace(q_start=i32(q_start), ctx_len=i32([s[0] for s in seqs]), token_seq=i32(token_seq),
+                           state_slot=i32([s[2] for s in seqs]), block_tables=tables.to(dev), num_seqs=len(seqs),
+                           max_query_len=max(s[1] for s in seqs), max_pages_used=width,
+                           max_page_id=int(tables.max()), max_state_slot=max(s[2] for s in seqs))
+
+
+@torch.inference_mode()
+def kernel_table(width: int = 2048, heads: int = 16, kv_heads: int = 4, window: int = 1024, keep: int = 16,
+                 prefill_rows: int = 4096, decode_seqs: int = 64, decode_ctx: int = 2048, experts: int = 32,
+                 top: int = 2, ff: int = 1024) -> List[dict]:
+    from .. import _C
+    dev, bf = torch.device("cuda"), torch.bfloat16
+    d = width // heads
+    page = 16
+    rows: List[dict] = []
+    scale = d ** -0.5
+
+    # ------------------------------------------------------------------ attention
+    for phase, seqs in (("prefill", [(0, prefill_rows // 2, 0, None), (0, prefill_rows // 2, 1, None)]),
+                        ("decode", [(decode_ctx, 1, i, None) for i in range(decode_seqs)])):
+        total_pages, laid = 0, []
+        for ctx, n, slot, _ in seqs:
+            pages = -(-(ctx + n) // page)
+            laid.append((ctx, n, slot, list(range(total_pages, total_pages + pages))))
+            total_pages += pages
+        batch = _ragged(laid, dev)
+        T = sum(s[1] for s in laid)
+        kc = torch.randn(total_pages, page, kv_heads * d, device=dev).to(bf)
+        vc = torch.randn(total_pages, page, kv_heads * d, device=dev).to(bf)
+        q = torch.randn(T, heads * d, device=dev)
+        talk = torch.eye(heads, device=dev) + 0.1 * torch.randn(heads, heads, device=dev)
+        out = torch.empty(T, heads * d, dtype=bf, device=dev)
+        t = _time(lambda: _C.mixer_ops.window_attention(out, q, kc, vc, talk, batch, heads, kv_heads, d, d, scale, window,
+                                                        keep, tiled=phase == "prefill"))
+        pairs = sum(min(c + i + 1, window + keep) for c, n, _, _ in laid for i in range(n))      # (query, key) pairs
+        keys = sum(min(c + n, (window + keep) if phase == "decode" else c + n) for c, n, _, _ in laid)
+        flops = 2.0 * pairs * heads * (d + kv_heads * d)
+        nbytes = keys * kv_heads * d * 2 * 2 + T * heads * d * (4 + 2)
+        rows.append(_row("window_attention (talking heads)", phase, t, nbytes, flops,
+                         MFMA_BF16 if phase == "prefill" else VALU_F32))
+        # the Llama path's kernel at the same head geometry
+        if phase == "prefill":
+            qh = torch.randn(T, heads, d, device=dev).to(bf)
+            kh = torch.randn(T, kv_heads, d, device=dev).to(bf)
+            vh = torch.randn(T, kv_heads, d, device=dev).to(bf)
+            oh = torch.empty_like(qh)
+            starts = torch.tensor([0, T // 2], dtype=torch.int32, device=dev)
+            lens = torch.tensor([T // 2, T // 2], dtype=torch.int32, device=dev)
+            t2 = _time(lambda: _C.ops.prefill_attention(oh, qh, kh, vh, starts, lens, T // 2, scale, None, window))
+            pairs2 = sum(min(i + 1, window) for i in range(T // 2)) * 2
+            rows.append(_row("prefill_attention (sliding window)", phase, t2, T * (heads + 2 * kv_heads) * d * 2 + T * heads * d * 2,
+                             4.0 * pairs2 * heads * d, MFMA_BF16, like="window_attention"))
+        else:
+            x = 8
+            nb = decode_seqs * (-(-window // page)) + 1
+            kc2 = torch.randn(nb, kv_heads, d // x, page, x, device=dev).to(bf)
+            vc2 = torch.randn(nb, kv_heads, d, page, device=dev).to(bf)
+            bt = torch.randperm(nb - 1, device=dev).to(torch.int32).view(decode_seqs, -1).contiguous()
+            cl = torch.full((decode_seqs,), window, dtype=torch.int32, device=dev)
+            qh = torch.randn(decode_seqs, heads, d, device=dev).to(bf)
+            oh = torch.empty_like(qh)
+            t2 = _time(lambda: _C.ops.paged_attention_v1(oh, qh, kc2, vc2, kv_heads, scale, bt, cl, page, window, None, "auto"))
+            rows.append(_row("paged_attention_v1 (window's worth of context)", phase, t2,
+                             decode_seqs * window * kv_heads * d * 2 * 2 + 2 * decode_seqs * heads * d * 2,
+                             4.0 * decode_seqs * window * heads * d, VALU_F32, like="window_attention"))
+
+    # ------------------------------------------------------------------ delta rules, convolution, gates
+    for phase, seqs in (("prefill", [(0, prefill_rows // 2, 0, []), (0, prefill_rows // 2, 1, [])]),
+                        ("decode", [(decode_ctx, 1, i, []) for i in range(decode_seqs)])):
+        batch = _ragged(seqs, dev)
+        T, B = sum(s[1] for s in seqs), len(seqs)
+        slots = max(B, 2)
+        # channel-decay rule: heads x [d, d]
+        qkv = torch.randn(T, 3 * heads * d, device=dev)
+        beta = torch.randn(T, heads, device=dev).to(bf)
+        decay = torch.randn(T, heads * d, device=dev).to(bf)
+        state = torch.zeros(slots, heads, d, d, device=dev)
+        o = torch.empty(T, heads * d, device=dev)
+        dt_bias, a_log = torch.zeros(heads * d, device=dev), torch.zeros(heads, device=dev)
+        t = _time(lambda: _C.mixer_ops.channel_delta(o, qkv, beta, decay, dt_bias, a_log, state, batch, heads, heads, d, d))
+        nbytes = T * (3 * heads * d * 4 + heads * d * 2 + heads * d * 4) + 2 * B * heads * d * d * 4
+        rows.append(_row("channel_delta", phase, t, nbytes, 8.0 * T * heads * d * d, VALU_F32))
+        # general rule: 2 * heads x [d / 2, d / 2]
+        h2, d2 = 2 * heads, d // 2
+        proj = torch.randn(T, 5 * h2 * d2, device=dev).to(bf)
+        n = h2 * d2
+        wpre = torch.randn(T, n, device=dev).to(bf)
+        state2 = torch.zeros(slots, h2, d2, d2, device=dev)
+        o2 = torch.empty(T, n, device=dev)
+        zeros = torch.zeros(n, device=dev)
+        t = _time(lambda: _C.mixer_ops.general_delta(o2, proj[:, :n], proj[:, n:2 * n], proj[:, 2 * n:3 * n], wpre, zeros,
+                                                     proj[:, 4 * n:], zeros, state2, batch, h2, d2))
+        rows.append(_row("general_delta", phase, t, T * n * (5 * 2 + 4) + 2 * B * h2 * d2 * d2 * 4, 9.0 * T * h2 * d2 * d2,
+                         VALU_F32))
+        # short convolution over q | k | v channels
+        ch = 3 * heads * d
+        xin = torch.randn(T, ch, device=dev).to(bf)
+        taps = torch.randn(ch, 4, device=dev)
+        cstate = torch.zeros(slots, 3, ch, device=dev)
+        cout = torch.empty(T, ch, device=dev)
+        t = _time(lambda: _C.mixer_ops.short_conv(cout, xin, taps, cstate, batch))
+        rows.append(_row("short_conv (+ state advance)", phase, t, T * ch * (2 + 4) + 2 * B * 3 * ch * 4, 8.0 * T * ch, VALU_F32))
+        # per-head norm and gate
+        gate = torch.randn(T, heads * d, device=dev).to(bf)
+        wn = torch.ones(d, device=dev)
+        g_out = torch.empty(T, heads * d, dtype=bf, device=dev)
+        t = _time(lambda: _C.mixer_ops.head_norm_gate(g_out, o, gate, wn, False, 1e-6, heads, d))
+        rows.append(_row("head_norm_gate", phase, t, T * heads * d * (4 + 2 + 2), 6.0 * T * heads * d, VALU_F32))
+        # norm of a sublayer's output added to the fp32 stream  /  Llama's fused add + norm
+        res = torch.randn(T, width, device=dev)
+        y = torch.randn(T, width, device=dev).to(bf)
+        cast = torch.empty(T, width, dtype=bf, device=dev)
+        gain = torch.ones(1, device=dev)
+        t = _time(lambda: _C.mixer_ops.scalar_norm_add(res, y, gain, 1e-6, cast))
+        rows.append(_row("scalar_norm_add (fp32 stream)", phase, t, T * width * (2 + 4 + 4 + 2), 4.0 * T * width, VALU_F32))
+        xr, rr, wr = y.clone(), y.clone(), torch.ones(width, dtype=bf, device=dev)
+        t = _time(lambda: _C.ops.fused_add_rms_norm(xr, rr, wr, 1e-6))
+        rows.append(_row("fused_add_rms_norm (bf16 stream)", phase, t, T * width * 2 * 4, 4.0 * T * width, VALU_F32,
+                         like="scalar_norm_add"))
+        # experts against a dense feed-forward of the same active size
+        hin = torch.randn(T, width, device=dev).to(bf)
+        up = torch.randn(experts, ff, width, device=dev).to(bf) * 0.02
+        down = torch.randn(experts, width, ff, device=dev).to(bf) * 0.02
+        choice = torch.rand(T, experts, device=dev).argsort(1)[:, :top].reshape(-1)
+        order = torch.sort(choice, stable=True).indices.to(torch.int32)
+        start = torch.zeros(experts + 1, dtype=torch.int32, device=dev)
+        start[1:] = torch.cumsum(torch.bincount(choice, minlength=experts), 0)
+        eo = torch.zeros(T, width, device=dev)
+        t = _time(lambda: _C.mixer_ops.expert_ffn(eo, hin, up, down, order, start, top, 1.0 / top))
+        flops = 4.0 * T * top * ff * width
+        touched = min(experts, T * top)
+        nbytes = touched * 2 * ff * width * 2 + T * width * (2 + 4) + T * top * ff * 2 * 2
+        rows.append(_row("expert_ffn (grouped, gelu)", phase, t, nbytes, flops, MFMA_BF16))
+        w1 = torch.randn(top * ff, width, device=dev).to(bf) * 0.02
+        w2 = torch.randn(width, top * ff, device=dev).to(bf) * 0.02
+        t = _time(lambda: torch.nn.functional.linear(torch.nn.functional.gelu(torch.nn.functional.linear(hin, w1)), w2))
+        rows.append(_row("dense feed-forward of the same active size (library GEMMs)", phase, t,
+                         2 * top * ff * width * 2 + T * width * 4 + T * top * ff * 4, flops, MFMA_BF16, like="expert_ffn"))
+    return rows
+
+
+def run(sizes=("2k",), with_kernels: bool = True) -> dict:
+    result = {"engine": {}, "kernels": {}}
+    for size in sizes:
+        pair = {}
+        for family in ("nepevik", "llama"):
+            pair[family] = {k: round(v, 2) for k, v in engine_throughput(f"{family}-{size}").items()}
+        result["engine"][size] = pair
+    if with_kernels:
+        result["kernels"]["2k"] = kernel_table()
+    return result
