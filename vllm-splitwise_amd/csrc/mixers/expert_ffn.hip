@@ -1,6 +1,7 @@
 // Feed-forward experts over rows that were sorted by expert: two grouped "NT" GEMMs (both operands
 // contiguous along the reduction), the first with the exact gelu as its epilogue, the second scattering
-// its rows back and adding them into an fp32 output.
+// its rows back and adding them into an fp32 output.  bf16 runs on the matrix cores (second half of this
+// file); fp32 -- true fp32, no reduced-precision matrix mode -- on LDS-tiled vector FMAs.
 //
 // The host does not know how many rows an expert got (the sort stays on the device), so the grid has the
 // upper bound ceil(pairs / TM) + experts row tiles and each workgroup finds its (expert, tile) from the
@@ -13,16 +14,16 @@ constexpr int TM = 32, TN = 64, TK = 32, kFfnThreads = 256;
 
 __device__ __forceinline__ float gelu_erf(float z) { return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f)); }
 
-// -> expert and first sorted row of this workgroup's tile, rows in it (0: nothing to do)
+// -> expert and first sorted row of this workgroup's tile of `tm` rows, rows in it (0: nothing to do)
 __device__ __forceinline__ int find_tile(const int32_t* __restrict__ expert_start, int num_experts, int tile,
-                                         int* expert, int* row0) {
+                                         int* expert, int* row0, int tm = TM) {
   for (int e = 0; e < num_experts; ++e) {
     const int lo = expert_start[e], n = expert_start[e + 1] - lo;
-    const int tiles = (n + TM - 1) / TM;
+    const int tiles = (n + tm - 1) / tm;
     if (tile < tiles) {
       *expert = e;
-      *row0 = lo + tile * TM;
-      return min(TM, n - tile * TM);
+      *row0 = lo + tile * tm;
+      return min(tm, n - tile * tm);
     }
     tile -= tiles;
   }
@@ -129,6 +130,95 @@ __global__ __launch_bounds__(kFfnThreads) void expert_down_kernel(
   }
 }
 
+
+// ------------------------------------------------------------------------------- bf16 on the matrix cores
+// 64 x 64 output tile per workgroup, one 32 x 32 quadrant per wave (v_mfma_f32_32x32x16_bf16, fp32 accumulation);
+// stages of 64 reduction steps go global -> LDS as 16-byte vectors.  Both operands are contiguous along the
+// reduction and are read with the SAME lane -> k mapping (8 consecutive k per lane, the wave's halves 8 apart),
+// so only the accumulator's layout matters: element i of lane l is row 8 * (i / 4) + 4 * (l / 32) + i % 4,
+// column l % 32.  Needs the reduction size to be a multiple of 8.
+constexpr int MM = 64, MN = 64, MK = 64, MPAD = 8;
+using bf16x8 = __attribute__((ext_vector_type(8))) __bf16;
+using f32x16 = __attribute__((ext_vector_type(16))) float;
+
+template <typename RowOf>
+__device__ __forceinline__ void tile_gemm_mfma(f32x16& acc, const uint16_t* __restrict__ a, RowOf a_row, int rows,
+                                               const uint16_t* __restrict__ b, int64_t b_off, int n0, int N, int K,
+                                               uint16_t (*As)[MK + MPAD], uint16_t (*Bs)[MK + MPAD]) {
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int wm = wave >> 1, wn = wave & 1;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+  for (int k0 = 0; k0 < K; k0 += MK) {
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+      const int e = tid + it * kFfnThreads, r = e >> 3, k = (e & 7) * 8;
+      uint4 va = make_uint4(0u, 0u, 0u, 0u), vb = make_uint4(0u, 0u, 0u, 0u);
+      if (r < rows && k0 + k < K) va = *reinterpret_cast<const uint4*>(a + a_row(r) * (int64_t)K + k0 + k);
+      if (n0 + r < N && k0 + k < K) vb = *reinterpret_cast<const uint4*>(b + b_off + (int64_t)(n0 + r) * K + k0 + k);
+      *reinterpret_cast<uint4*>(&As[r][k]) = va;
+      *reinterpret_cast<uint4*>(&Bs[r][k]) = vb;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int ks = 0; ks < MK; ks += 16) {
+      const bf16x8 av = *reinterpret_cast<const bf16x8*>(&As[wm * 32 + (lane & 31)][ks + 8 * (lane >> 5)]);
+      const bf16x8 bv = *reinterpret_cast<const bf16x8*>(&Bs[wn * 32 + (lane & 31)][ks + 8 * (lane >> 5)]);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, bv, acc, 0, 0, 0);
+    }
+    __syncthreads();
+  }
+}
+
+// calls f(row in tile, column in tile, value) for the 16 accumulator elements of this lane
+template <typename F>
+__device__ __forceinline__ void for_each_acc(const f32x16& acc, F&& f) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wm = wave >> 1, wn = wave & 1;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) f(wm * 32 + 8 * (i / 4) + 4 * (lane >> 5) + (i % 4), wn * 32 + (lane & 31), acc[i]);
+}
+
+__global__ __launch_bounds__(kFfnThreads) void expert_up_gelu_mfma_kernel(
+    uint16_t* __restrict__ hidden, const uint16_t* __restrict__ x, const uint16_t* __restrict__ up,
+    const int32_t* __restrict__ order, const int32_t* __restrict__ expert_start, int num_experts, int width, int ff,
+    int top) {
+  __shared__ __attribute__((aligned(16))) uint16_t As[MM][MK + MPAD];
+  __shared__ __attribute__((aligned(16))) uint16_t Bs[MN][MK + MPAD];
+  int e, row0;
+  const int rows = find_tile(expert_start, num_experts, blockIdx.x, &e, &row0, MM);
+  if (rows == 0) return;
+  const int n0 = blockIdx.y * MN;
+  f32x16 acc;
+  tile_gemm_mfma(acc, x, [&](int r) { return (int64_t)(order[row0 + r] / top); }, rows, up, (int64_t)e * ff * width, n0,
+                 ff, width, As, Bs);
+  for_each_acc(acc, [&](int r, int c, float v) {
+    if (r < rows && n0 + c < ff) hidden[(int64_t)(row0 + r) * ff + n0 + c] = sw::float_to_bf16_bits(gelu_erf(v));
+  });
+}
+
+__global__ __launch_bounds__(kFfnThreads) void expert_down_mfma_kernel(
+    float* __restrict__ out, const uint16_t* __restrict__ hidden, const uint16_t* __restrict__ down,
+    const int32_t* __restrict__ order, const int32_t* __restrict__ expert_start, int num_experts, int width, int ff,
+    int top, float weight) {
+  __shared__ __attribute__((aligned(16))) uint16_t As[MM][MK + MPAD];
+  __shared__ __attribute__((aligned(16))) uint16_t Bs[MN][MK + MPAD];
+  int e, row0;
+  const int rows = find_tile(expert_start, num_experts, blockIdx.x, &e, &row0, MM);
+  if (rows == 0) return;
+  const int n0 = blockIdx.y * MN;
+  f32x16 acc;
+  tile_gemm_mfma(acc, hidden, [&](int r) { return (int64_t)(row0 + r); }, rows, down, (int64_t)e * width * ff, n0, width,
+                 ff, As, Bs);
+  for_each_acc(acc, [&](int r, int c, float v) {
+    if (r < rows && n0 + c < width) {
+      float* p = out + (int64_t)(order[row0 + r] / top) * width + n0 + c;
+      if (top == 1) *p += weight * v;
+      else atomicAdd(p, weight * v);
+    }
+  });
+}
+
 }  // namespace swm
 
 extern "C" {
@@ -140,6 +230,14 @@ int swm_expert_up_gelu(void* hidden, const void* x, const void* up, const int32_
   if (sorted_rows == 0) return SW_OK;
   SW_CHECK_ARG(act_ok(act_dtype), "expert_up_gelu: unsupported dtype %d", act_dtype);
   SW_CHECK_ARG(num_experts > 0 && width > 0 && ff > 0 && top > 0 && sorted_rows < (1ll << 30), "expert_up_gelu: bad shape");
+  if (act_dtype == SW_BF16 && width % 8 == 0) {
+    const dim3 mgrid((unsigned)((sorted_rows + MM - 1) / MM + num_experts), (unsigned)((ff + MN - 1) / MN));
+    hipLaunchKernelGGL(expert_up_gelu_mfma_kernel, mgrid, dim3(kFfnThreads), 0, static_cast<hipStream_t>(stream),
+                       static_cast<uint16_t*>(hidden), static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(up),
+                       order, expert_start, num_experts, width, ff, top);
+    SW_CHECK_LAUNCH();
+    return SW_OK;
+  }
   const dim3 grid((unsigned)((sorted_rows + TM - 1) / TM + num_experts), (unsigned)((ff + TN - 1) / TN));
   SWM_DISPATCH_ACT(act_dtype, hipLaunchKernelGGL(expert_up_gelu_kernel<T>, grid, dim3(kFfnThreads), 0,
                                                  static_cast<hipStream_t>(stream), hidden, x, up, order, expert_start,
@@ -155,6 +253,14 @@ int swm_expert_down(float* out, const void* hidden, const void* down, const int3
   if (sorted_rows == 0) return SW_OK;
   SW_CHECK_ARG(act_ok(act_dtype), "expert_down: unsupported dtype %d", act_dtype);
   SW_CHECK_ARG(num_experts > 0 && width > 0 && ff > 0 && top > 0 && sorted_rows < (1ll << 30), "expert_down: bad shape");
+  if (act_dtype == SW_BF16 && ff % 8 == 0) {
+    const dim3 mgrid((unsigned)((sorted_rows + MM - 1) / MM + num_experts), (unsigned)((width + MN - 1) / MN));
+    hipLaunchKernelGGL(expert_down_mfma_kernel, mgrid, dim3(kFfnThreads), 0, static_cast<hipStream_t>(stream), out,
+                       static_cast<const uint16_t*>(hidden), static_cast<const uint16_t*>(down), order, expert_start,
+                       num_experts, width, ff, top, weight);
+    SW_CHECK_LAUNCH();
+    return SW_OK;
+  }
   const dim3 grid((unsigned)((sorted_rows + TM - 1) / TM + num_experts), (unsigned)((width + TN - 1) / TN));
   SWM_DISPATCH_ACT(act_dtype, hipLaunchKernelGGL(expert_down_kernel<T>, grid, dim3(kFfnThreads), 0,
                                                  static_cast<hipStream_t>(stream), out, hidden, down, order,
