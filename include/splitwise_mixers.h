@@ -57,13 +57,15 @@ int swm_qk_norm_cache(float* q_out, const void* q, const void* k, const void* v,
  * sum_g talk[h, g] * weights_g and are applied to the values of h's own key/value head.
  * q fp32 [rows, heads * dim]; caches [pages * page_size, kv_heads * dim | vdim] act_dtype;
  * talk fp32 [heads, heads]; out act_dtype [rows, heads * vdim].
- * `tiled` != 0 picks the kernel that shares staged keys among 16 consecutive queries of a sequence
- * (prompt portions); 0 the one-token-per-workgroup kernel (decode steps). */
+ * `splits` > 1 (steps of few tokens): every token's visible keys are cut into that many runs, one workgroup
+ * each, joined by a second launch; `partial` then holds rows * splits * (2 * heads + heads * kv_heads * vdim)
+ * floats of scratch. */
 int swm_window_attention(void* out, const float* q, const void* key_cache, const void* value_cache,
                          const float* talk, const int32_t* block_tables, int table_width,
                          const int32_t* q_start, const int32_t* ctx_len, const int32_t* token_seq,
                          int64_t rows, int num_seqs, int heads, int kv_heads, int dim, int vdim, int page_size,
-                         float scale, int window, int keep_first, int tiled, int act_dtype, void* stream);
+                         float scale, int window, int keep_first, int splits, float* partial, int act_dtype,
+                         void* stream);
 
 /* Short causal convolution over time per channel, then silu.  x act_dtype [rows, channels] (row stride
  * x_stride); taps fp32 [channels, num_taps], last column = current token; state fp32

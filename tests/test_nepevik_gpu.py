@@ -115,7 +115,7 @@ def _attention_oracle(q, k, v, H, G, d, dv, window, keep, scale, talk, qn, kn, e
 
 @pytest.mark.parametrize("H,G,d,dv,window,keep", [(4, 2, 16, 32, 8, 3), (6, 6, 8, 8, 5, 0), (3, 1, 24, 72, 17, 1),
                                                   (8, 4, 32, 130, 40, 6)])
-@pytest.mark.parametrize("mode", ["prompt", "decode", "portions"])
+@pytest.mark.parametrize("mode", ["prompt", "decode", "portions", "decode_split"])
 def test_window_attention_edges(H, G, d, dv, window, keep, mode):
     """Keys just inside and just outside the window, the last kept first token and the one after it, a key far
     back, keys on both sides of a page border -- as a whole prompt, decoded one by one, and in portions; pages
@@ -145,7 +145,9 @@ def test_window_attention_edges(H, G, d, dv, window, keep, mode):
     vc = torch.full((pool, page, G * dv), 50.0, device=DEV)
     proj = torch.cat([q, k, v], 1).to(DEV)
     nq, nk = H * d, G * d
-    portions = {"prompt": [n], "decode": [n - 12] + [1] * 12, "portions": [2, 3, window, 1, 2, page + 1]}[mode]
+    portions = {"prompt": [n], "decode": [n - 12] + [1] * 12, "portions": [2, 3, window, 1, 2, page + 1],
+                "decode_split": [n - 12] + [1] * 12}[mode]
+    splits = {"decode_split": 3, "portions": 2}.get(mode)              # runs of keys joined by a second launch
     portions = portions + ([n - sum(portions)] if sum(portions) < n else [])
     outs, done = [], 0
     for m in portions:
@@ -156,7 +158,7 @@ def test_window_attention_edges(H, G, d, dv, window, keep, mode):
                                    kc, vc, slots)
         out = torch.empty(m, H * dv, dtype=torch.float32, device=DEV)
         _C.mixer_ops.window_attention(out, q32, kc, vc, talk.to(DEV), ragged([(done, m, 0, table)]), H, G, d, dv, scale,
-                                      window, keep, tiled=m > 1)
+                                      window, keep, splits=splits)
         outs.append(out)
         done += m
     got = torch.cat(outs).double().cpu()

@@ -29,7 +29,7 @@ _SIGNATURES = {
     "swm_scalar_norm": [_p, _p, _p, _f, _l, _i, _i, _p],
     "swm_qk_norm_cache": [_p, _p, _p, _p, _l, _p, _p, _f, _p, _p, _p, _l, _i, _i, _i, _i, _p],
     "swm_window_attention": [_p, _p, _p, _p, _p, _p, _i, _p, _p, _p, _l, _i, _i, _i, _i, _i, _i, _f, _i, _i, _i,
-                             _i, _p],
+                             _p, _i, _p],
     "swm_short_conv": [_p, _p, _l, _p, _p, _p, _p, _p, _p, _l, _i, _i, _i, _p],
     "swm_short_conv_advance": [_p, _p, _l, _p, _p, _p, _i, _i, _i, _i, _p],
     "swm_channel_delta": [_p, _p, _p, _l, _p, _p, _p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p, _i, _p],
@@ -182,8 +182,10 @@ def _ragged_ok(batch, rows: int) -> int:
 
 def window_attention(out: torch.Tensor, q: torch.Tensor, key_cache: torch.Tensor, value_cache: torch.Tensor,
                      talk: torch.Tensor, batch, heads: int, kv_heads: int, dim: int, vdim: int, scale: float,
-                     window: int, keep_first: int, tiled: bool = False) -> None:
-    """out [rows, heads * vdim] (cache dtype); q fp32 [rows, heads * dim]; caches [pages, page, kv_heads * size]."""
+                     window: int, keep_first: int, splits: Optional[int] = None) -> None:
+    """out [rows, heads * vdim] (cache dtype); q fp32 [rows, heads * dim]; caches [pages, page, kv_heads * size].
+    ``splits``: runs that a token's keys are cut into (default: enough to fill the GPU when the step has few
+    tokens, 1 otherwise)."""
     _dev(out, q, key_cache, value_cache, talk)
     _f32c(q, "q")
     _f32c(talk, "talk")
@@ -200,12 +202,18 @@ def window_attention(out: torch.Tensor, q: torch.Tensor, key_cache: torch.Tensor
           "window_attention: shapes")
     _need(batch.max_pages_used <= tables.shape[1] and batch.max_page_id < key_cache.shape[0],
           "window_attention: block tables exceed the cache")
+    if splits is None:
+        most_keys = min(window + keep_first, batch.max_pages_used * key_cache.shape[1])
+        splits = max(1, min(8, 512 // rows, most_keys // 64))
+    partial = None
+    if splits > 1:
+        partial = torch.empty(rows * splits * (2 * heads + heads * kv_heads * vdim), dtype=torch.float32, device=q.device)
     with torch.cuda.device(q.device):
         _check(load_library().swm_window_attention(
             out.data_ptr(), q.data_ptr(), key_cache.data_ptr(), value_cache.data_ptr(), talk.data_ptr(),
             tables.data_ptr(), tables.shape[1], batch.q_start.data_ptr(), batch.ctx_len.data_ptr(),
             batch.token_seq.data_ptr(), rows, n, heads, kv_heads, dim, vdim, key_cache.shape[1], scale, window,
-            keep_first, int(tiled), _act(out), _stream(q)))
+            keep_first, splits, None if partial is None else partial.data_ptr(), _act(out), _stream(q)))
 
 
 def short_conv(out: torch.Tensor, x: torch.Tensor, taps: torch.Tensor, state: torch.Tensor, batch) -> None:

@@ -138,13 +138,13 @@ def kernel_table(width: int = 2048, heads: int = 16, kv_heads: int = 4, window: 
         talk = torch.eye(heads, device=dev) + 0.1 * torch.randn(heads, heads, device=dev)
         out = torch.empty(T, heads * d, dtype=bf, device=dev)
         t = _time(lambda: _C.mixer_ops.window_attention(out, q, kc, vc, talk, batch, heads, kv_heads, d, d, scale, window,
-                                                        keep, tiled=phase == "prefill"))
+                                                        keep))
         pairs = sum(min(c + i + 1, window + keep) for c, n, _, _ in laid for i in range(n))      # (query, key) pairs
         keys = sum(min(c + n, (window + keep) if phase == "decode" else c + n) for c, n, _, _ in laid)
         flops = 2.0 * pairs * heads * (d + kv_heads * d)
         nbytes = keys * kv_heads * d * 2 * 2 + T * heads * d * (4 + 2)
         rows.append(_row("window_attention (talking heads)", phase, t, nbytes, flops,
-                         MFMA_BF16 if phase == "prefill" else VALU_F32))
+                         VALU_F32))            # its weights stay fp32: the bf16 matrix path is closed to it
         # the Llama path's kernel at the same head geometry
         if phase == "prefill":
             qh = torch.randn(T, heads, d, device=dev).to(bf)

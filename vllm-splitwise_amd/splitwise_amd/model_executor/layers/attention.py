@@ -258,6 +258,5 @@ class WindowTalkingAttention(nn.Module):
                                        value_cache, md.slot_mapping)
         out = torch.empty(rows, self.heads * self.vdim, dtype=q.dtype, device=q.device)
         _C.mixer_ops.window_attention(out, q32, key_cache, value_cache, self.talk.data, md.ragged, self.heads,
-                                      self.kv_heads, self.dim, self.vdim, self.scale, self.window, self.keep_first,
-                                      tiled=md.ragged.max_query_len > 1)
+                                      self.kv_heads, self.dim, self.vdim, self.scale, self.window, self.keep_first)
         return out
