@@ -9,8 +9,8 @@
 // key-side vector (S^T k, S^T q) is a per-lane partial sum over its rows plus two xor-shuffles; no LDS, no
 // barriers, so the only serial dependence is the recurrence itself.  The state is read once at the first token
 // of the step (not at all when the sequence starts here) and written once after the last: a decode step moves
-// exactly the state, a prompt portion moves it once per portion.  The next token's operands are fetched
-// (float4 loads) before the current token's arithmetic.
+// exactly the state, a prompt portion moves it once per portion.  Operands of the next 8 tokens are in flight
+// while the current 8 are worked through (see delta_recurrence_kernel).
 #include "mixers_common.cuh"
 
 namespace swm {
@@ -18,9 +18,17 @@ namespace swm {
 constexpr int kColsPerWave = 16;
 constexpr int kPrepThreads = 256;
 
-__device__ __forceinline__ float group_sum(float v) {      // over the 4 lanes of a column
-  v += __shfl_xor(v, 1, 64);
-  v += __shfl_xor(v, 2, 64);
+// sum over the 4 lanes of a column (a quad): DPP quad permutes, no trip through the LDS crossbar
+__device__ __forceinline__ float quad_swap(float v, int ctrl_is_xor2) {
+  const int x = __float_as_int(v);
+  // quad_perm [1,0,3,2] = 0xB1 swaps neighbours, [2,3,0,1] = 0x4E swaps pairs
+  const int y = ctrl_is_xor2 ? __builtin_amdgcn_update_dpp(0, x, 0x4E, 0xF, 0xF, true)
+                             : __builtin_amdgcn_update_dpp(0, x, 0xB1, 0xF, 0xF, true);
+  return __int_as_float(y);
+}
+__device__ __forceinline__ float group_sum(float v) {
+  v += quad_swap(v, 0);
+  v += quad_swap(v, 1);
   return v;
 }
 
@@ -53,11 +61,14 @@ __global__ __launch_bounds__(kPrepThreads) void channel_delta_prep_kernel(
     kk = sw::wave_sum(kk);
     const float qf = qscale / sqrtf(qq + 1e-6f), kf = 1.0f / sqrtf(kk + 1e-6f);
     const float rate = expf(a_log[h]);
-    float* o = ops + (t * heads + h) * 3 * (int64_t)dim;
-    for (int i = lane; i < dim; i += 64) {
-      o[i] = q[i] * qf;
-      o[dim + i] = k[i] * kf;
-      o[2 * dim + i] = expf(-rate * softplusf_(ld<T>(decay_pre, (t * heads + h) * (int64_t)dim + i) + dt_bias[h * dim + i]));
+    const int dimp = (dim + 3) & ~3;                     // operand rows are padded to whole 16-byte pieces
+    float* o = ops + (t * heads + h) * 3 * (int64_t)dimp;
+    for (int i = lane; i < dimp; i += 64) {
+      const bool in = i < dim;
+      o[i] = in ? q[i] * qf : 0.0f;
+      o[dimp + i] = in ? k[i] * kf : 0.0f;
+      o[2 * dimp + i] = in ? expf(-rate * softplusf_(ld<T>(decay_pre, (t * heads + h) * (int64_t)dim + i) + dt_bias[h * dim + i]))
+                           : 0.0f;
     }
     if (lane == 0) beta[t * heads + h] = sigmoidf_(ld<T>(beta_pre, t * beta_stride + h));
   }
@@ -81,89 +92,177 @@ __global__ __launch_bounds__(kPrepThreads) void general_delta_prep_kernel(
     }
     kk = sw::wave_sum(kk);
     const float inv = 1.0f / (kk + 1e-6f);
-    float* o = ops + (t * heads + h) * 4 * (int64_t)dim;
-    for (int i = lane; i < dim; i += 64) {
-      const float k = ld<T>(kp, t * rkv_stride + h * dim + i);
-      o[i] = ld<T>(rp, t * rkv_stride + h * dim + i);
-      o[dim + i] = k;
-      o[2 * dim + i] = expf(-kDecay * sigmoidf_(ld<T>(decay_pre, t * decay_stride + h * dim + i) + w0[h * dim + i]));
-      o[3 * dim + i] = sigmoidf_(ld<T>(rate_pre, t * rate_stride + h * dim + i) + a_bias[h * dim + i]) * k * inv;
+    const int dimp = (dim + 3) & ~3;
+    float* o = ops + (t * heads + h) * 4 * (int64_t)dimp;
+    for (int i = lane; i < dimp; i += 64) {
+      const bool in = i < dim;
+      const float k = in ? ld<T>(kp, t * rkv_stride + h * dim + i) : 0.0f;
+      o[i] = in ? ld<T>(rp, t * rkv_stride + h * dim + i) : 0.0f;
+      o[dimp + i] = k;
+      o[2 * dimp + i] = in ? expf(-kDecay * sigmoidf_(ld<T>(decay_pre, t * decay_stride + h * dim + i) + w0[h * dim + i])) : 0.0f;
+      o[3 * dimp + i] = in ? sigmoidf_(ld<T>(rate_pre, t * rate_stride + h * dim + i) + a_bias[h * dim + i]) * k * inv : 0.0f;
     }
   }
 }
 
 // ---------------------------------------------------------------------------------------- recurrences
 // RQ rows per lane (a multiple of 4; dim <= 4 * RQ): lane group rg holds rows [rg * RQ, (rg + 1) * RQ).
-// NOPS operand vectors of `dim` floats per (token, head), read as float4 when dim is a multiple of 4.
-template <int RQ, int NOPS>
-struct Operands {
-  float v[NOPS][RQ];
-  __device__ __forceinline__ void fetch(const float* __restrict__ base, int dim, int row0) {
-    if ((dim & 3) == 0) {
-#pragma unroll
-      for (int a = 0; a < NOPS; ++a)
-#pragma unroll
-        for (int i = 0; i < RQ; i += 4) {
-          float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
-          if (row0 + i < dim) x = *reinterpret_cast<const float4*>(base + a * dim + row0 + i);
-          v[a][i] = x.x; v[a][i + 1] = x.y; v[a][i + 2] = x.z; v[a][i + 3] = x.w;
-        }
-    } else {
-#pragma unroll
-      for (int a = 0; a < NOPS; ++a)
-#pragma unroll
-        for (int i = 0; i < RQ; ++i) v[a][i] = row0 + i < dim ? base[a * dim + row0 + i] : 0.0f;
-    }
-  }
-};
+// One recurrence kernel for both rules.  MODE 0 (channel): operands {q, k, g}, v fp32 from the convolution's
+// output, beta;  MODE 1 (general): operands {r, k, w, a k / |k|^2}, v in the activation type TV.
+//
+// Operands reach the lanes through LDS in chunks of kChunk (a multiple of 4) tokens: while the wave works through one chunk, the
+// loads of the next are in flight (each lane fetches a different 16-byte piece, so a chunk costs a handful of
+// loads per lane instead of a broadcast load per operand row), and a token step reads its rows from LDS.
+constexpr int kChunk = 4;
 
-template <int RQ>
-__global__ __launch_bounds__(64) void channel_delta_kernel(
-    float* __restrict__ out, const float* __restrict__ ops, const float* __restrict__ beta,
-    const float* __restrict__ qkv, float* __restrict__ state, const int32_t* __restrict__ q_start,
-    const int32_t* __restrict__ ctx_len, const int32_t* __restrict__ state_slot, int heads, int kv_heads, int dim,
-    int vdim) {
+template <int RQ, int NOPS, int MODE, typename TV>
+__global__ __launch_bounds__(64) void delta_recurrence_kernel(
+    float* __restrict__ out, const float* __restrict__ ops, const float* __restrict__ beta, const void* __restrict__ vsrc,
+    int64_t v_stride, int64_t v_off, float* __restrict__ state, const int32_t* __restrict__ q_start,
+    const int32_t* __restrict__ ctx_len, const int32_t* __restrict__ state_slot, int heads, int dim, int vdim) {
+  constexpr int PIECES = (kChunk * NOPS * RQ + 63) / 64;        // 16-byte pieces of a chunk per lane (dim <= 4 RQ)
+  extern __shared__ float lds[];
+  constexpr int RQ4 = 4 * RQ;                                    // an operand row in LDS: padded with zeros
+  const int dimp = (dim + 3) & ~3;
+  const int tok_floats = NOPS * dimp;                            // operand floats of one (token, head) in memory
+  constexpr int lds_floats = NOPS * RQ4;                         // ... and in LDS
+  constexpr int tok_stride = lds_floats + 20;                    // + 16 values + beta, kept on 16 bytes
   const int lane = threadIdx.x, rg = lane & 3, row0 = rg * RQ;
-  const int col = blockIdx.x * kColsPerWave + (lane >> 2);
+  for (int e = lane; e < 2 * kChunk * tok_stride; e += 64) lds[e] = 0.0f;      // the padding stays zero
+  __syncthreads();
+  const int cw = lane >> 2;
+  const int col = blockIdx.x * kColsPerWave + cw;
   const int h = blockIdx.y, s = blockIdx.z;
   const int first = q_start[s], n = q_start[s + 1] - first;
   if (n == 0) return;
   const bool col_ok = col < vdim;
   const int colc = col_ok ? col : vdim - 1;             // out-of-range lanes shadow the last column, never store
-  const int64_t row_w = 2 * (int64_t)kv_heads * dim + (int64_t)heads * vdim;
-  const int64_t v_off = 2 * (int64_t)kv_heads * dim + (int64_t)h * vdim + colc;
   float* S = state + ((int64_t)state_slot[s] * heads + h) * dim * vdim;
   float Sr[RQ];
 #pragma unroll
   for (int i = 0; i < RQ; ++i) Sr[i] = (ctx_len[s] > 0 && row0 + i < dim) ? S[(int64_t)(row0 + i) * vdim + colc] : 0.0f;
-  Operands<RQ, 3> nxt;
-  float vn, bn;
-  auto fetch = [&](int t) {
-    nxt.fetch(ops + ((int64_t)t * heads + h) * 3 * dim, dim, row0);
-    vn = qkv[(int64_t)t * row_w + v_off];
-    bn = beta[(int64_t)t * heads + h];
+  const int pieces_per_tok = tok_floats / 4;
+  float4 held[PIECES];
+  float vheld[kChunk / 4] = {0.0f}, bheld = 0.0f;
+  // a lane's share of chunk `c`: global -> registers
+  auto fetch = [&](int c) {
+    const int t0 = first + c * kChunk, left = min(kChunk, first + n - t0);
+    const int count = left * pieces_per_tok;
+#pragma unroll
+    for (int j = 0; j < PIECES; ++j) {
+      const int idx = lane + 64 * j;
+      if (idx < count)
+        held[j] = *reinterpret_cast<const float4*>(ops + ((int64_t)(t0 + idx / pieces_per_tok) * heads + h) * tok_floats +
+                                                   4 * (idx % pieces_per_tok));
+    }
+#pragma unroll
+    for (int j = 0; j < kChunk / 4; ++j) {
+      const int tk = (lane >> 4) + 4 * j, cc = min((int)blockIdx.x * kColsPerWave + (lane & 15), vdim - 1);
+      if (tk < left) vheld[j] = ld<TV>(vsrc, (int64_t)(t0 + tk) * v_stride + v_off + (int64_t)h * vdim + cc);
+    }
+    if (MODE == 0 && lane < left) bheld = beta[(int64_t)(t0 + lane) * heads + h];
   };
-  fetch(first);
-  for (int t = first; t < first + n; ++t) {
-    const Operands<RQ, 3> cur = nxt;
-    const float v = vn, b = bn;
-    if (t + 1 < first + n) fetch(t + 1);
-    float ks = 0.0f;
+  // registers -> LDS buffer
+  auto park = [&](int c, float* buf) {
+    const int t0 = first + c * kChunk, left = min(kChunk, first + n - t0);
+    const int count = left * pieces_per_tok;
 #pragma unroll
-    for (int i = 0; i < RQ; ++i) {
-      Sr[i] *= cur.v[2][i];
-      ks += cur.v[1][i] * Sr[i];
+    for (int j = 0; j < PIECES; ++j) {
+      const int idx = lane + 64 * j;
+      if (idx < count) {
+        const int off = idx % pieces_per_tok, per_row = dimp / 4;
+        *reinterpret_cast<float4*>(buf + (idx / pieces_per_tok) * tok_stride + (off / per_row) * RQ4 + 4 * (off % per_row)) =
+            held[j];
+      }
     }
-    ks = group_sum(ks);
-    const float u = b * (v - ks);
-    float o = 0.0f;
 #pragma unroll
-    for (int i = 0; i < RQ; ++i) {
-      Sr[i] += cur.v[1][i] * u;
-      o += cur.v[0][i] * Sr[i];
+    for (int j = 0; j < kChunk / 4; ++j) {
+      const int tk = (lane >> 4) + 4 * j;
+      if (tk < left) buf[tk * tok_stride + lds_floats + (lane & 15)] = vheld[j];
     }
-    o = group_sum(o);
-    if (rg == 0 && col_ok) out[((int64_t)t * heads + h) * vdim + col] = o;
+    if (MODE == 0 && lane < left) buf[lane * tok_stride + lds_floats + 16] = bheld;
+  };
+  const int chunks = (n + kChunk - 1) / kChunk;
+  const int buf_floats = kChunk * tok_stride;          // two buffers, used in turn
+  fetch(0);
+  park(0, lds);
+  __syncthreads();
+#pragma unroll 1
+  for (int c = 0; c < chunks; ++c) {
+    if (c + 1 < chunks) fetch(c + 1);
+    const float* buf = lds + (c & 1) * buf_floats;
+    const int t0 = first + c * kChunk, left = min(kChunk, first + n - t0);
+    // Two register sets take turns: while one token is worked through, the next one's operand rows are on
+    // their way from LDS (the reads are issued first and waited for a whole token step later).
+    auto rows_in = [&](float4 (&dst)[NOPS][RQ / 4], float& v, float& b, int tk) {
+      const float* op = buf + tk * tok_stride + row0;
+#pragma unroll
+      for (int a = 0; a < NOPS; ++a)
+#pragma unroll
+        for (int i = 0; i < RQ / 4; ++i)
+          dst[a][i] = *reinterpret_cast<const float4*>(op + a * RQ4 + 4 * i);
+      v = buf[tk * tok_stride + lds_floats + cw];
+      if (MODE == 0) b = buf[tk * tok_stride + lds_floats + 16];
+    };
+    auto step = [&](const float4 (&x)[NOPS][RQ / 4], float v, float b, int tk) {
+      float o = 0.0f, ks = 0.0f;
+      if (MODE == 0) {                                   // x: q, k, g
+#pragma unroll
+        for (int i = 0; i < RQ / 4; ++i) {
+          {
+            const float4 k4 = x[1][i], g4 = x[2][i];
+            Sr[4 * i] *= g4.x; Sr[4 * i + 1] *= g4.y; Sr[4 * i + 2] *= g4.z; Sr[4 * i + 3] *= g4.w;
+            ks += k4.x * Sr[4 * i] + k4.y * Sr[4 * i + 1] + k4.z * Sr[4 * i + 2] + k4.w * Sr[4 * i + 3];
+          }
+        }
+        ks = group_sum(ks);
+        const float u = b * (v - ks);
+#pragma unroll
+        for (int i = 0; i < RQ / 4; ++i) {
+          {
+            const float4 q4 = x[0][i], k4 = x[1][i];
+            Sr[4 * i] += k4.x * u; Sr[4 * i + 1] += k4.y * u; Sr[4 * i + 2] += k4.z * u; Sr[4 * i + 3] += k4.w * u;
+            o += q4.x * Sr[4 * i] + q4.y * Sr[4 * i + 1] + q4.z * Sr[4 * i + 2] + q4.w * Sr[4 * i + 3];
+          }
+        }
+      } else {                                           // x: r, k, w, a k / |k|^2
+#pragma unroll
+        for (int i = 0; i < RQ / 4; ++i) {
+          {
+            const float4 k4 = x[1][i];
+            ks += k4.x * Sr[4 * i] + k4.y * Sr[4 * i + 1] + k4.z * Sr[4 * i + 2] + k4.w * Sr[4 * i + 3];
+          }
+        }
+        ks = group_sum(ks);                              // k^T S of the OLD state
+#pragma unroll
+        for (int i = 0; i < RQ / 4; ++i) {
+          {
+            const float4 r4 = x[0][i], k4 = x[1][i], w4 = x[2][i], a4 = x[NOPS - 1][i];
+            Sr[4 * i] = w4.x * Sr[4 * i] - a4.x * ks + k4.x * v;
+            Sr[4 * i + 1] = w4.y * Sr[4 * i + 1] - a4.y * ks + k4.y * v;
+            Sr[4 * i + 2] = w4.z * Sr[4 * i + 2] - a4.z * ks + k4.z * v;
+            Sr[4 * i + 3] = w4.w * Sr[4 * i + 3] - a4.w * ks + k4.w * v;
+            o += r4.x * Sr[4 * i] + r4.y * Sr[4 * i + 1] + r4.z * Sr[4 * i + 2] + r4.w * Sr[4 * i + 3];
+          }
+        }
+      }
+      o = group_sum(o);
+      if (rg == 0 && col_ok) out[((int64_t)(t0 + tk) * heads + h) * vdim + col] = o;
+    };
+    float4 xa[NOPS][RQ / 4], xb[NOPS][RQ / 4];
+    float va = 0.0f, vb = 0.0f, ba = 0.0f, bb = 0.0f;
+    rows_in(xa, va, ba, 0);
+#pragma unroll 1
+    for (int tk = 0; tk < left; tk += 2) {
+      if (tk + 1 < left) rows_in(xb, vb, bb, tk + 1);
+      step(xa, va, ba, tk);
+      if (tk + 1 < left) {
+        if (tk + 2 < left) rows_in(xa, va, ba, tk + 2);
+        step(xb, vb, bb, tk + 1);
+      }
+    }
+    if (c + 1 < chunks) park(c + 1, lds + ((c + 1) & 1) * buf_floats);
+    __syncthreads();
   }
   if (col_ok) {
 #pragma unroll
@@ -172,51 +271,13 @@ __global__ __launch_bounds__(64) void channel_delta_kernel(
   }
 }
 
-template <typename T, int RQ>
-__global__ __launch_bounds__(64) void general_delta_kernel(
-    float* __restrict__ out, const float* __restrict__ ops, const void* __restrict__ vp, int64_t v_stride,
-    float* __restrict__ state, const int32_t* __restrict__ q_start, const int32_t* __restrict__ ctx_len,
-    const int32_t* __restrict__ state_slot, int heads, int dim) {
-  const int lane = threadIdx.x, rg = lane & 3, row0 = rg * RQ;
-  const int col = blockIdx.x * kColsPerWave + (lane >> 2);
-  const int h = blockIdx.y, s = blockIdx.z;
-  const int first = q_start[s], n = q_start[s + 1] - first;
-  if (n == 0) return;
-  const bool col_ok = col < dim;
-  const int colc = col_ok ? col : dim - 1;
-  float* S = state + ((int64_t)state_slot[s] * heads + h) * dim * dim;
-  float Sr[RQ];
-#pragma unroll
-  for (int i = 0; i < RQ; ++i) Sr[i] = (ctx_len[s] > 0 && row0 + i < dim) ? S[(int64_t)(row0 + i) * dim + colc] : 0.0f;
-  Operands<RQ, 4> nxt;
-  float vn;
-  auto fetch = [&](int t) {
-    nxt.fetch(ops + ((int64_t)t * heads + h) * 4 * dim, dim, row0);
-    vn = ld<T>(vp, (int64_t)t * v_stride + h * dim + colc);
-  };
-  fetch(first);
-  for (int t = first; t < first + n; ++t) {
-    const Operands<RQ, 4> cur = nxt;
-    const float v = vn;
-    if (t + 1 < first + n) fetch(t + 1);
-    float ks = 0.0f;
-#pragma unroll
-    for (int i = 0; i < RQ; ++i) ks += cur.v[1][i] * Sr[i];
-    ks = group_sum(ks);                                  // k^T S of the OLD state
-    float o = 0.0f;
-#pragma unroll
-    for (int i = 0; i < RQ; ++i) {
-      Sr[i] = cur.v[2][i] * Sr[i] - cur.v[3][i] * ks + cur.v[1][i] * v;
-      o += cur.v[0][i] * Sr[i];
-    }
-    o = group_sum(o);
-    if (rg == 0 && col_ok) out[((int64_t)t * heads + h) * dim + col] = o;
-  }
-  if (col_ok) {
-#pragma unroll
-    for (int i = 0; i < RQ; ++i)
-      if (row0 + i < dim) S[(int64_t)(row0 + i) * dim + col] = Sr[i];
-  }
+inline size_t recurrence_lds_bytes(int nops, int rq) { return sizeof(float) * 2 * kChunk * (size_t)(nops * 4 * rq + 20); }
+
+// launches above 64 KiB of LDS (key sizes near 256) have to be allowed first
+template <typename K>
+inline hipError_t allow_lds(K kernel, size_t bytes) {
+  if (bytes <= 64 * 1024) return hipSuccess;
+  return hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
 }
 
 }  // namespace swm
@@ -233,8 +294,12 @@ __global__ __launch_bounds__(64) void general_delta_kernel(
 
 extern "C" {
 
-int64_t swm_channel_delta_workspace_floats(int64_t rows, int heads, int dim) { return rows * heads * (3 * (int64_t)dim + 1); }
-int64_t swm_general_delta_workspace_floats(int64_t rows, int heads, int dim) { return rows * heads * 4 * (int64_t)dim; }
+int64_t swm_channel_delta_workspace_floats(int64_t rows, int heads, int dim) {
+  return rows * heads * (3 * (int64_t)((dim + 3) & ~3) + 1);
+}
+int64_t swm_general_delta_workspace_floats(int64_t rows, int heads, int dim) {
+  return rows * heads * 4 * (int64_t)((dim + 3) & ~3);
+}
 
 int swm_channel_delta(float* out, const float* qkv, const void* beta_pre, int64_t beta_stride,
                       const void* decay_pre, const float* dt_bias, const float* a_log, float* state,
@@ -250,14 +315,18 @@ int swm_channel_delta(float* out, const float* qkv, const void* beta_pre, int64_
                vdim);
   hipStream_t s = static_cast<hipStream_t>(stream);
   float* ops = workspace;
-  float* beta = workspace + rows * heads * 3 * (int64_t)dim;
+  float* beta = workspace + rows * heads * 3 * (int64_t)((dim + 3) & ~3);
   SWM_DISPATCH_ACT(act_dtype, hipLaunchKernelGGL(channel_delta_prep_kernel<T>, dim3((unsigned)rows), dim3(kPrepThreads), 0,
                                                  s, ops, beta, qkv, beta_pre, beta_stride, decay_pre, dt_bias, a_log,
                                                  heads, kv_heads, dim, vdim););
   SW_CHECK_LAUNCH();
   const dim3 grid((unsigned)((vdim + kColsPerWave - 1) / kColsPerWave), (unsigned)heads, (unsigned)num_seqs);
-  SWM_DISPATCH_ROWS(dim, hipLaunchKernelGGL((channel_delta_kernel<RQ>), grid, dim3(64), 0, s, out, ops, beta, qkv, state,
-                                            q_start, ctx_len, state_slot, heads, kv_heads, dim, vdim););
+  const int64_t row_w = 2 * (int64_t)kv_heads * dim + (int64_t)heads * vdim;
+  SWM_DISPATCH_ROWS(dim, SW_CHECK_HIP(allow_lds(delta_recurrence_kernel<RQ, 3, 0, float>, recurrence_lds_bytes(3, RQ))););
+  SWM_DISPATCH_ROWS(dim, hipLaunchKernelGGL((delta_recurrence_kernel<RQ, 3, 0, float>), grid, dim3(64),
+                                            recurrence_lds_bytes(3, RQ), s, out, ops, beta, qkv, row_w,
+                                            2 * (int64_t)kv_heads * dim, state, q_start, ctx_len, state_slot, heads, dim,
+                                            vdim););
   SW_CHECK_LAUNCH();
   return SW_OK;
 }
@@ -278,9 +347,11 @@ int swm_general_delta(float* out, const void* r, const void* k, const void* v, i
                                                  rate_stride, a_bias, heads, dim););
   SW_CHECK_LAUNCH();
   const dim3 grid((unsigned)((dim + kColsPerWave - 1) / kColsPerWave), (unsigned)heads, (unsigned)num_seqs);
-  SWM_DISPATCH_ACT(act_dtype, SWM_DISPATCH_ROWS(dim, hipLaunchKernelGGL((general_delta_kernel<T, RQ>), grid, dim3(64), 0, s,
-                                                                        out, workspace, v, rkv_stride, state, q_start,
-                                                                        ctx_len, state_slot, heads, dim);););
+  SWM_DISPATCH_ACT(act_dtype, SWM_DISPATCH_ROWS(dim, SW_CHECK_HIP(allow_lds(delta_recurrence_kernel<RQ, 4, 1, T>,
+                                                                            recurrence_lds_bytes(4, RQ)));););
+  SWM_DISPATCH_ACT(act_dtype, SWM_DISPATCH_ROWS(dim, hipLaunchKernelGGL(
+      (delta_recurrence_kernel<RQ, 4, 1, T>), grid, dim3(64), recurrence_lds_bytes(4, RQ), s, out, workspace, nullptr, v,
+      rkv_stride, (int64_t)0, state, q_start, ctx_len, state_slot, heads, dim, dim);););
   SW_CHECK_LAUNCH();
   return SW_OK;
 }

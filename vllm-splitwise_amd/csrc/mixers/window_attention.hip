@@ -410,9 +410,11 @@ int launch_staged(void* out, const float* q, const void* key_cache, const void* 
                   float scale, int window, int keep_first, int splits, float* partial, hipStream_t stream) {
   const size_t lds = staged_lds_bytes(heads, kv_heads, dim, vdim);
   auto kernel = window_attention_staged_kernel<T, GMAX, NR>;
-  if (lds > 64 * 1024) {
+  static thread_local size_t allowed = 64 * 1024;       // what this instantiation may use so far
+  if (lds > allowed) {
     SW_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                      (int)lds));
+    allowed = lds;
   }
   hipLaunchKernelGGL(kernel, dim3((unsigned)rows, (unsigned)splits), dim3(kAttnThreads), lds, stream, out, q, key_cache,
                      value_cache, talk, block_tables, table_width, q_start, ctx_len, token_seq, heads, kv_heads, dim,
@@ -421,9 +423,11 @@ int launch_staged(void* out, const float* q, const void* key_cache, const void* 
   if (splits > 1) {
     const size_t jl = sizeof(float) * ((size_t)splits * heads + 4 + (size_t)heads * kv_heads * vdim);
     auto join = window_attention_join_kernel<T>;
-    if (jl > 64 * 1024) {
+    static thread_local size_t join_allowed = 64 * 1024;
+    if (jl > join_allowed) {
       SW_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(join), hipFuncAttributeMaxDynamicSharedMemorySize,
                                        (int)jl));
+      join_allowed = jl;
     }
     hipLaunchKernelGGL(join, dim3((unsigned)rows), dim3(kAttnThreads), jl, stream, out, partial, talk, splits, heads,
                        kv_heads, vdim);
@@ -439,9 +443,11 @@ int launch_token(void* out, const float* q, const void* key_cache, const void* v
                  float scale, int window, int keep_first, hipStream_t stream) {
   const size_t lds = sizeof(float) * ((size_t)heads * dim + (size_t)heads * kv_heads * vdim);
   auto kernel = window_attention_token_kernel<T, GMAX, NV>;
-  if (lds > 64 * 1024) {
+  static thread_local size_t allowed = 64 * 1024;
+  if (lds > allowed) {
     SW_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                      (int)lds));
+    allowed = lds;
   }
   hipLaunchKernelGGL(kernel, dim3((unsigned)rows), dim3(kAttnThreads), lds, stream, out, q, key_cache, value_cache,
                      talk, block_tables, table_width, q_start, ctx_len, token_seq, heads, kv_heads, dim, vdim,

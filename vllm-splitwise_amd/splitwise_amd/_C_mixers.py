@@ -257,7 +257,7 @@ def channel_delta(out: torch.Tensor, qkv: torch.Tensor, beta_pre: torch.Tensor, 
             out.data_ptr(), qkv.data_ptr(), beta_pre.data_ptr(), _rows(beta_pre, "beta_pre"), decay_pre.data_ptr(),
             dt_bias.data_ptr(), a_log.data_ptr(), state.data_ptr(), batch.q_start.data_ptr(),
             batch.ctx_len.data_ptr(), batch.state_slot.data_ptr(), rows, n, heads, kv_heads, dim, vdim,
-            torch.empty(rows * heads * (3 * dim + 1), dtype=torch.float32, device=qkv.device).data_ptr(),
+            torch.empty(rows * heads * (3 * (-(-dim // 4) * 4) + 1), dtype=torch.float32, device=qkv.device).data_ptr(),
             _act(decay_pre), _stream(qkv)))
 
 
@@ -281,7 +281,7 @@ def general_delta(out: torch.Tensor, r: torch.Tensor, k: torch.Tensor, v: torch.
             _rows(decay_pre, "decay_pre"), w0.data_ptr(), rate_pre.data_ptr(), _rows(rate_pre, "rate_pre"),
             a_bias.data_ptr(), state.data_ptr(), batch.q_start.data_ptr(), batch.ctx_len.data_ptr(),
             batch.state_slot.data_ptr(), rows, n, heads, dim,
-            torch.empty(rows * heads * 4 * dim, dtype=torch.float32, device=r.device).data_ptr(), _act(r),
+            torch.empty(rows * heads * 4 * (-(-dim // 4) * 4), dtype=torch.float32, device=r.device).data_ptr(), _act(r),
             _stream(r)))
 
 
