@@ -128,8 +128,10 @@ __global__ __launch_bounds__(64) void delta_recurrence_kernel(
   constexpr int lds_floats = NOPS * RQ4;                         // ... and in LDS
   constexpr int tok_stride = lds_floats + 20;                    // + 16 values + beta, kept on 16 bytes
   const int lane = threadIdx.x, rg = lane & 3, row0 = rg * RQ;
-  for (int e = lane; e < 2 * kChunk * tok_stride; e += 64) lds[e] = 0.0f;      // the padding stays zero
-  __syncthreads();
+  if (dimp < RQ4) {                                              // rows shorter than their LDS slot: the padding is
+    for (int e = lane; e < 2 * kChunk * tok_stride; e += 64) lds[e] = 0.0f;    // zeroed once and never written
+    __syncthreads();
+  }
   const int cw = lane >> 2;
   const int col = blockIdx.x * kColsPerWave + cw;
   const int h = blockIdx.y, s = blockIdx.z;

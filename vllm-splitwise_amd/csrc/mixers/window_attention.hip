@@ -146,7 +146,7 @@ __global__ __launch_bounds__(kAttnThreads) void window_attention_token_kernel(
 // ------------------------------------------------------------------------------------------ staged kernel
 // One workgroup per new token, all heads together.  A tile of 16 keys and their values (every key/value head) is
 // staged ONCE in LDS as fp32 and shared by all heads: scores by threads (head, key), the running softmax by one
-// thread per head, the value accumulation by threads (head, 8 value channels) for all key/value heads.  Needs
+// thread per head, the value accumulation by threads (head, 4 + 4 value channels) for all key/value heads.  Needs
 // key size % 4 == 0, value size % 8 == 0 and whole 16-byte vectors per cached row; other shapes take the
 // kernel above.
 constexpr int kTileKeys = 16;
@@ -300,8 +300,9 @@ __global__ __launch_bounds__(kAttnThreads) void window_attention_staged_kernel(
 #pragma unroll
         for (int c = 0; c < GMAX; ++c) {
           if (c < kv_heads) {
-            const float4* vv = reinterpret_cast<const float4*>(v_lds + k * vrow + c * vdim + ch * 8);
-            const float4 a = vv[0], b = vv[1];
+            // channels 4 ch .. 4 ch + 3 of each half of the head: 16 lanes read 256 contiguous bytes
+            const float* vr = v_lds + k * vrow + c * vdim + ch * 4;
+            const float4 a = *reinterpret_cast<const float4*>(vr), b = *reinterpret_cast<const float4*>(vr + vdim / 2);
             acc[r][c][0] += w * a.x; acc[r][c][1] += w * a.y; acc[r][c][2] += w * a.z; acc[r][c][3] += w * a.w;
             acc[r][c][4] += w * b.x; acc[r][c][5] += w * b.y; acc[r][c][6] += w * b.z; acc[r][c][7] += w * b.w;
           }
@@ -327,7 +328,8 @@ __global__ __launch_bounds__(kAttnThreads) void window_attention_staged_kernel(
       for (int c = 0; c < GMAX; ++c)
         if (c < kv_heads)
 #pragma unroll
-          for (int x = 0; x < 8; ++x) dst[2 * heads + ((int64_t)g * kv_heads + c) * vdim + ch * 8 + x] = acc[r][c][x];
+          for (int x = 0; x < 8; ++x)
+            dst[2 * heads + ((int64_t)g * kv_heads + c) * vdim + (x < 4 ? 0 : vdim / 2) + ch * 4 + (x & 3)] = acc[r][c][x];
     }
     return;
   }
@@ -341,7 +343,8 @@ __global__ __launch_bounds__(kAttnThreads) void window_attention_staged_kernel(
     for (int c = 0; c < GMAX; ++c)
       if (c < kv_heads)
 #pragma unroll
-        for (int x = 0; x < 8; ++x) mixed[((int64_t)g * kv_heads + c) * vdim + ch * 8 + x] = acc[r][c][x] * inv;
+        for (int x = 0; x < 8; ++x)
+          mixed[((int64_t)g * kv_heads + c) * vdim + (x < 4 ? 0 : vdim / 2) + ch * 4 + (x & 3)] = acc[r][c][x] * inv;
   }
   __syncthreads();
   for (int e = threadIdx.x; e < heads * vdim; e += kAttnThreads) {
