@@ -398,3 +398,35 @@ def test_greedy_generation_through_the_entry_point(models, name):
             assert row[tok] >= row.max() - 1e-3 * (row.max() - row.min()), (k, tok, int(row.argmax()))
     sched = llm.llm_engine.scheduler
     assert sched.state_slots.num_free() == 3 and not sched.running and not sched.waiting
+
+
+def test_trace_run_replays_a_schedule(models, tmp_path):
+    """``bin/trace_run`` as a user starts it: steps on standard input, ``done <step>`` after each, logits files in
+    the order of the entries; requests that sit out a step, end, and hand their pages and slot on."""
+    import json
+    import os
+    import subprocess
+    import numpy as np
+    m = models["b"]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    a, b, c = m.reqs["r1"], m.reqs["r2"], m.reqs["r4"]
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": a[:7], "want": [0, 6]}, {"id": "b", "tokens": b[:2], "want": []}], "end": []},
+        {"step": 1, "entries": [{"id": "b", "tokens": b[2:], "want": [15]}, {"id": "a", "tokens": a[7:8], "want": [0]}], "end": ["b"]},
+        {"step": 2, "entries": [{"id": "a", "tokens": a[8:], "want": [len(a) - 9]}, {"id": "c", "tokens": c, "want": [0, len(c) - 1]}],
+         "end": ["a", "c"]},
+        {"step": 3, "entries": [{"id": "b", "tokens": b, "want": [len(b) - 1]}], "end": ["b"]},        # the name comes back
+    ]
+    out = tmp_path / "out"
+    proc = subprocess.run([os.path.join(root, "bin", "trace_run"), "--model", m.path, "--dtype", "float32", "--out", str(out),
+                           "--max-tokens", "128", "--max-requests", "2"],
+                          input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == [f"done {i}" for i in range(4)]
+    vocab = m.cfg["vocab"]
+    want = {0: [m.want["r1"][0], m.want["r1"][6]], 1: [m.want["r2"][17], m.want["r1"][7]],
+            2: [m.want["r1"][len(a) - 1], m.want["r4"][0], m.want["r4"][len(c) - 1]], 3: [m.want["r2"][len(b) - 1]]}
+    for step, rows in want.items():
+        got = torch.from_numpy(np.fromfile(out / f"{step}.f32", dtype="<f4").reshape(-1, vocab))
+        assert got.shape[0] == len(rows)
+        assert nu.row_error(got, torch.stack(rows)) < FP32_TOL, step

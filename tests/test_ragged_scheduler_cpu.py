@@ -134,3 +134,9 @@ def test_too_long_prompts_are_ignored():
     g, _ = add(sched, "a", 40, 0)
     metas, outs = sched.schedule()
     assert not metas and outs.ignored_seq_groups == [g]
+
+
+def test_trace_replay_refuses_models_without_ragged_steps(tmp_path):
+    """Exit code 3, at the start, for an architecture whose steps are not ragged."""
+    from splitwise_amd.entrypoints import trace_replay
+    assert trace_replay.main(["--model", "llama-tiny", "--dtype", "bfloat16", "--out", str(tmp_path), "--max-tokens", "64"]) == 3
