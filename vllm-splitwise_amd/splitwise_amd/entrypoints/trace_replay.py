@@ -75,6 +75,8 @@ def main(argv=None) -> int:
         plan, want = {}, {}
         for entry in step["entries"]:
             rid, tokens = str(entry["id"]), [int(t) for t in entry["tokens"]]
+            if not tokens:
+                continue                                   # nothing to run for this request in this step
             if rid in live:
                 engine.extend_request(rid, tokens)
             else:
@@ -83,10 +85,12 @@ def main(argv=None) -> int:
             plan[rid] = len(tokens)
             if entry.get("want"):
                 want[rid] = [int(p) for p in entry["want"]]
+                if min(want[rid]) < 0 or max(want[rid]) >= len(tokens):
+                    raise ValueError(f"step {step['step']}, request {rid}: a wanted place lies outside its tokens")
         if plan:
             logits = engine.step_planned(plan, want)
             if want:
-                rows = torch.cat([logits[str(e["id"])] for e in step["entries"] if e.get("want")], 0)
+                rows = torch.cat([logits[str(e["id"])] for e in step["entries"] if e.get("want") and e["tokens"]], 0)
                 data = rows.float().cpu().numpy().astype("<f4")
                 assert data.shape[1] == vocab
                 tmp = os.path.join(args.out, f".{step['step']}.part")
