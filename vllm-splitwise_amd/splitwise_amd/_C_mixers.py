@@ -81,6 +81,25 @@ def _stream(t: torch.Tensor) -> int:
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
+class _SameDevice:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_SAME_DEVICE = _SameDevice()
+
+
+def _on_device_of(t: torch.Tensor):
+    """Context that makes ``t``'s device current; free when it already is (an eager step makes some seventy
+    of these calls, and switching devices costs more than the launch)."""
+    if t.device.index == torch.cuda.current_device():
+        return _SAME_DEVICE
+    return torch.cuda.device(t.device)
+
+
 def _act(t: torch.Tensor) -> int:
     try:
         return _ACT[t.dtype]
@@ -119,7 +138,7 @@ def scalar_norm_add(residual: torch.Tensor, y: torch.Tensor, gain: torch.Tensor,
     stride = _rows(y, "y")
     if cast_out is not None:
         _need(cast_out.is_contiguous() and cast_out.shape == y.shape, "scalar_norm_add: cast_out")
-    with torch.cuda.device(y.device):
+    with _on_device_of(y):
         _check(load_library().swm_scalar_norm_add(
             residual.data_ptr(), y.data_ptr(), gain.data_ptr(), eps,
             None if cast_out is None else cast_out.data_ptr(), y.shape[0], y.shape[1], stride, _act(y),
@@ -131,7 +150,7 @@ def scalar_norm(out: torch.Tensor, x: torch.Tensor, gain: torch.Tensor, eps: flo
     _f32c(x, "x")
     _f32c(gain, "gain")
     _need(out.is_contiguous() and out.shape == x.shape and x.dim() == 2 and gain.numel() == 1, "scalar_norm: shapes")
-    with torch.cuda.device(x.device):
+    with _on_device_of(x):
         _check(load_library().swm_scalar_norm(out.data_ptr(), x.data_ptr(), gain.data_ptr(), eps, x.shape[0],
                                               x.shape[1], _act(out), _stream(x)))
 
@@ -162,7 +181,7 @@ def qk_norm_cache(q_out: torch.Tensor, q: torch.Tensor, k: Optional[torch.Tensor
               "qk_norm_cache: slot_mapping must be int64 [rows]")
         slots = key_cache.shape[0] * key_cache.shape[1]
         _need(value_cache.shape[0] * value_cache.shape[1] == slots, "qk_norm_cache: caches differ in slots")
-    with torch.cuda.device(q.device):
+    with _on_device_of(q):
         _check(load_library().swm_qk_norm_cache(
             q_out.data_ptr(), q.data_ptr(), None if k is None else k.data_ptr(), None if v is None else v.data_ptr(),
             stride, q_gain.data_ptr(), None if k is None else k_gain.data_ptr(), eps,
@@ -208,7 +227,7 @@ def window_attention(out: torch.Tensor, q: torch.Tensor, key_cache: torch.Tensor
     partial = None
     if splits > 1:
         partial = torch.empty(rows * splits * (2 * heads + heads * kv_heads * vdim), dtype=torch.float32, device=q.device)
-    with torch.cuda.device(q.device):
+    with _on_device_of(q):
         _check(load_library().swm_window_attention(
             out.data_ptr(), q.data_ptr(), key_cache.data_ptr(), value_cache.data_ptr(), talk.data_ptr(),
             tables.data_ptr(), tables.shape[1], batch.q_start.data_ptr(), batch.ctx_len.data_ptr(),
@@ -229,7 +248,7 @@ def short_conv(out: torch.Tensor, x: torch.Tensor, taps: torch.Tensor, state: to
     k = taps.shape[1]
     _need(out.shape == x.shape and taps.shape[0] == channels and state.shape[1:] == (k - 1, channels)
           and batch.max_state_slot < state.shape[0], "short_conv: shapes")
-    with torch.cuda.device(x.device):
+    with _on_device_of(x):
         lib = load_library()
         _check(lib.swm_short_conv(out.data_ptr(), x.data_ptr(), stride, taps.data_ptr(), state.data_ptr(),
                                   batch.q_start.data_ptr(), batch.ctx_len.data_ptr(), batch.token_seq.data_ptr(),
@@ -252,7 +271,7 @@ def channel_delta(out: torch.Tensor, qkv: torch.Tensor, beta_pre: torch.Tensor, 
           and decay_pre.dtype == beta_pre.dtype and dt_bias.numel() == heads * dim and a_log.numel() == heads
           and state.shape[1:] == (heads, dim, vdim) and batch.max_state_slot < state.shape[0],
           "channel_delta: shapes")
-    with torch.cuda.device(qkv.device):
+    with _on_device_of(qkv):
         _check(load_library().swm_channel_delta(
             out.data_ptr(), qkv.data_ptr(), beta_pre.data_ptr(), _rows(beta_pre, "beta_pre"), decay_pre.data_ptr(),
             dt_bias.data_ptr(), a_log.data_ptr(), state.data_ptr(), batch.q_start.data_ptr(),
@@ -275,7 +294,7 @@ def general_delta(out: torch.Tensor, r: torch.Tensor, k: torch.Tensor, v: torch.
           and _rows(k, "k") == stride and _rows(v, "v") == stride and out.shape == (rows, size)
           and w0.numel() == size and a_bias.numel() == size and state.shape[1:] == (heads, dim, dim)
           and batch.max_state_slot < state.shape[0], "general_delta: shapes")
-    with torch.cuda.device(r.device):
+    with _on_device_of(r):
         _check(load_library().swm_general_delta(
             out.data_ptr(), r.data_ptr(), k.data_ptr(), v.data_ptr(), stride, decay_pre.data_ptr(),
             _rows(decay_pre, "decay_pre"), w0.data_ptr(), rate_pre.data_ptr(), _rows(rate_pre, "rate_pre"),
@@ -295,7 +314,7 @@ def head_norm_gate(out: torch.Tensor, o: torch.Tensor, gate: torch.Tensor, weigh
     _need(o.shape == (rows, heads * vdim) and gate.shape == o.shape and out.shape == o.shape and out.is_contiguous()
           and out.dtype == gate.dtype and weight.numel() == (heads * vdim if per_head_weight else vdim),
           "head_norm_gate: shapes")
-    with torch.cuda.device(o.device):
+    with _on_device_of(o):
         _check(load_library().swm_head_norm_gate(out.data_ptr(), o.data_ptr(), gate.data_ptr(), _rows(gate, "gate"),
                                                  weight.data_ptr(), vdim if per_head_weight else 0, eps, rows, heads,
                                                  vdim, _act(out), _stream(o)))
@@ -316,7 +335,7 @@ def expert_ffn(out: torch.Tensor, x: torch.Tensor, up: torch.Tensor, down: torch
           and expert_start.is_contiguous(), "expert_ffn: shapes")
     pairs = rows * top
     hidden = torch.empty(pairs, ff, dtype=x.dtype, device=x.device)
-    with torch.cuda.device(x.device):
+    with _on_device_of(x):
         lib = load_library()
         _check(lib.swm_expert_up_gelu(hidden.data_ptr(), x.data_ptr(), up.data_ptr(), order.data_ptr(),
                                       expert_start.data_ptr(), experts, pairs, width, ff, top, _act(x), _stream(x)))

@@ -4,8 +4,8 @@
 expert weighs 1 / top.  An expert is down(gelu(up x)) with the exact (erf) gelu and no biases.  An optional
 shared expert of the same form runs for every token and is added after a per-token sigmoid gate.
 
-Rows are grouped by expert on the device (a stable sort of the (row, choice) pairs by expert id and a prefix
-sum of the counts), so each expert's rows are one contiguous run of a gathered matrix.
+Rows are grouped by expert on the device (a stable sort of the (row, choice) pairs by expert id, then a binary
+search for every expert's first pair), so each expert's rows are one contiguous run and the host never waits.
 """
 from typing import Dict, Optional
 
@@ -35,11 +35,11 @@ class TableRoutedExperts(nn.Module):
         """-> (order [rows * top] int32: pair index row * top + choice, sorted by expert;
                expert_start [experts + 1] int32)."""
         experts = self.table.data.index_select(0, token_ids).view(-1)              # [rows * top]
-        order = torch.sort(experts, stable=True).indices.to(torch.int32)
-        counts = torch.bincount(experts, minlength=self.num_experts)
-        start = torch.zeros(self.num_experts + 1, dtype=torch.int32, device=token_ids.device)
-        start[1:] = torch.cumsum(counts, 0)
-        return order, start
+        by_expert, order = torch.sort(experts, stable=True)
+        # first sorted pair of every expert: no count ever travels to the host
+        edges = torch.arange(self.num_experts + 1, dtype=experts.dtype, device=experts.device)
+        start = torch.searchsorted(by_expert, edges).to(torch.int32)
+        return order.to(torch.int32), start
 
     def forward(self, h: torch.Tensor, token_ids: torch.Tensor) -> torch.Tensor:
         """-> fp32 [rows, width]: the experts' sum is accumulated in fp32."""
