@@ -20,7 +20,6 @@ import json
 import os
 import sys
 
-import numpy as np
 import torch
 
 

@@ -17,7 +17,7 @@ import torch
 
 HBM_BPS = 8.0e12
 MFMA_BF16 = 2.5e15
-VALU_F32 = 157.0e12          # 256 CUs x 4 SIMDs x 16 lanes x 2 (fma) x 2 (dual issue not counted) x 2.4 GHz
+VALU_F32 = 157.0e12          # 256 CUs x 4 SIMDs x 16 lanes x 2 (fma) x 2 (packed pairs) x 2.4 GHz: the published vector peak
 
 
 def _sync() -> None:
