@@ -20,7 +20,11 @@ import json
 import os
 import sys
 
-import torch
+# fp32 means fp32 whatever the caller's environment says: these are read when torch (or the BLAS library) loads
+for _name in ("TORCH_ALLOW_TF32_CUBLAS_OVERRIDE", "HIPBLASLT_ALLOW_TF32", "ROCBLAS_XF32_XDL_MATH_OP"):
+    os.environ.pop(_name, None)
+
+import torch  # noqa: E402
 
 
 def _ensure_built(architecture_needs_mixers: bool) -> None:
