@@ -4,7 +4,9 @@
  * Operators of decoders that mix tokens by other means than rotary softmax attention over a full
  * context: recurrent delta-rule layers with a per-sequence state, short causal convolutions,
  * attention over a sliding window plus kept first tokens with the heads' weights mixed after the
- * softmax, and norms with a single gain.  A library of its own so that a model that needs only
+ * softmax, norms with a single gain; linear attention with a decay per head, soft-capped gated attention
+ * with partial rotary embedding, routed experts with group-limited choice, and the fused residual-add + norm
+ * of layers whose sublayers run side by side.  A library of its own so that a model that needs only
  * these compiles only these.
  *
  * A step is a RAGGED batch: the new tokens of all sequences back to back in one token dimension.
@@ -30,7 +32,7 @@
 extern "C" {
 #endif
 
-#define SWM_ABI_VERSION 1
+#define SWM_ABI_VERSION 2
 int swm_abi_version(void);
 const char* swm_last_error(void);
 
@@ -126,6 +128,72 @@ int swm_expert_up_gelu(void* hidden, const void* x, const void* up, const int32_
 int swm_expert_down(float* out, const void* hidden, const void* down, const int32_t* order,
                     const int32_t* expert_start, int num_experts, int64_t sorted_rows, int width, int ff,
                     int top, float weight, int act_dtype, void* stream);
+
+/* The same two steps with the hidden layer's activation named (SWM_ACT_GELU: exact gelu, SWM_ACT_RELU2: the square
+ * of relu) and with a weight per (row, choice) pair: out[row] += weight * pair_weight[row * top + choice] * ...
+ * (pair_weight fp32 [rows * top], NULL: all 1). */
+#define SWM_ACT_GELU 0
+#define SWM_ACT_RELU2 1
+int swm_expert_up(void* hidden, const void* x, const void* up, const int32_t* order, const int32_t* expert_start,
+                  int num_experts, int64_t sorted_rows, int width, int ff, int top, int activation, int act_dtype,
+                  void* stream);
+int swm_expert_down_weighted(float* out, const void* hidden, const void* down, const int32_t* order,
+                             const int32_t* expert_start, int num_experts, int64_t sorted_rows, int width, int ff,
+                             int top, float weight, const float* pair_weight, int act_dtype, void* stream);
+
+/* ---- layers whose two sublayers read one norm of an fp32 residual stream ---- */
+
+/* residual[t] += a[t] + b[t] + c[t] (each may be NULL; a, b act_dtype with row strides, c fp32 contiguous; the
+ * addends are summed first), then, when `out` is not NULL,
+ * out[t] = act_dtype(residual[t] / sqrt(mean(residual[t]^2) + eps) * (offset + weight)), weight fp32 [width]. */
+int swm_stream_add_norm(float* residual, const void* a, int64_t a_stride, const void* b, int64_t b_stride,
+                        const float* c, const float* weight, float offset, float eps, void* out, int64_t rows,
+                        int width, int act_dtype, void* stream);
+
+/* in [rows, 2 * ff] = gate | up (row stride in_stride):  g = min(gate, limit), u = clamp(up, -limit, limit),
+ * out[rows, ff] = g * sigmoid(alpha * g) * (u + shift).  limit may be +inf. */
+int swm_clamped_glu(void* out, const void* in, int64_t in_stride, int64_t rows, int ff, float alpha, float limit,
+                    float shift, int act_dtype, void* stream);
+/* out[rows, ff] = max(in, 0)^2 */
+int swm_relu2(void* out, const void* in, int64_t in_stride, int64_t rows, int ff, int act_dtype, void* stream);
+
+/* Rotary embedding on neighbouring pairs (2i, 2i + 1) of the first rot_dims coordinates of every head, angle
+ * = float(positions[t]) * inv_freq[i] in fp32 (inv_freq fp32 [rot_dims / 2]); the other coordinates pass.
+ * q_out fp32 [rows, heads * dim] = rotated q.  With k != NULL: key_cache[slot] = rotated k, value_cache[slot] = v
+ * (slot = slot_mapping[t], < 0: not cached; caches [slots, kv_heads * dim | vdim] act_dtype).  q, k, v are column
+ * ranges of one projection output (row stride in_stride). */
+int swm_rope_cache(float* q_out, const void* q, const void* k, const void* v, int64_t in_stride,
+                   const int64_t* positions, const float* inv_freq, int rot_dims, void* key_cache, void* value_cache,
+                   const int64_t* slot_mapping, int64_t rows, int heads, int kv_heads, int dim, int vdim, int act_dtype,
+                   void* stream);
+
+/* Router of a mixture of experts: s = sigmoid(router h) in fp32 (router fp32 [experts, width]); choice scores
+ * s + correction (NULL: none); experts form `groups` equal groups of neighbours, a group scores the sum of its two
+ * largest choice scores and only the best `keep` groups stay in the choice (groups == 1 or keep == groups: all);
+ * the `top` largest choice scores are chosen; weights = s of the chosen / (their sum + 1e-20) * scale.
+ * chosen int32 [rows, top], weights fp32 [rows, top]. */
+int swm_group_router(int32_t* chosen, float* weights, const void* h, int64_t h_stride, const float* router,
+                     const float* correction, int64_t rows, int width, int experts, int top, int groups, int keep,
+                     float scale, int act_dtype, void* stream);
+
+/* Causal softmax attention of every new token over its sequence's paged keys with grouped query heads (query head
+ * h reads key/value head h / (heads / kv_heads)): score = (q . k) * scale, then softcap * tanh(score / softcap) when
+ * softcap > 0; position i sees j <= i (and i - j < window when window > 0); fp32 scores, weights and sums.
+ * q fp32 [rows, heads * dim] (already rotated); caches [pages * page_size, kv_heads * dim | vdim] act_dtype;
+ * gate (NULL: none) act_dtype [rows, heads * vdim] with row stride: the output is multiplied by sigmoid(gate);
+ * out act_dtype [rows, heads * vdim]. */
+int swm_capped_attention(void* out, const float* q, const void* key_cache, const void* value_cache,
+                         const void* gate, int64_t gate_stride, const int32_t* block_tables, int table_width,
+                         const int32_t* q_start, const int32_t* ctx_len, int64_t rows, int num_seqs, int heads,
+                         int kv_heads, int dim, int vdim, int page_size, float scale, float softcap, int window,
+                         int act_dtype, void* stream);
+
+/* Linear attention with one decay per head:  S <- decay[h] S + k v^T;  o = S^T q, with q, k, v = silu of the given
+ * projections (act_dtype, column ranges of one output with row stride in_stride; q, k [rows, heads * dim],
+ * v [rows, heads * vdim]); decay fp32 [heads]; state fp32 [slots, heads, dim, vdim]; out fp32 [rows, heads * vdim]. */
+int swm_lightning(float* out, const void* q, const void* k, const void* v, int64_t in_stride, const float* decay,
+                  float* state, const int32_t* q_start, const int32_t* ctx_len, const int32_t* state_slot, int64_t rows,
+                  int num_seqs, int heads, int dim, int vdim, int act_dtype, void* stream);
 
 #ifdef __cplusplus
 }

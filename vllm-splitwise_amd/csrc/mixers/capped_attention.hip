@@ -1,0 +1,305 @@
+// Causal softmax attention of a ragged step over paged keys with grouped query heads, an optional soft cap on the
+// scores (cap * tanh(score / cap)), an optional sliding window and an optional sigmoid gate on the output.
+// Scores, softmax weights and the weighted sum of values are fp32: both products run on the matrix cores in
+// fp32 (v_mfma_f32_32x32x2_f32), keys and values are widened when they come from a bf16 cache.
+//
+// Work split.  A tile is 32 query rows of ONE sequence and ONE key/value head: the R = heads / kv_heads query heads
+// of that group for 32 / R consecutive new tokens (row = token * R + head), so a decode step keeps all heads of a
+// group in one tile and a prompt shares every loaded key among R * tokens rows.  A workgroup of NW waves owns a
+// tile; wave w takes the 32-key tiles w, w + NW, ... of the visible keys with a running softmax of its own, and
+// the waves are joined through LDS in a fixed order (results do not depend on timing).
+//
+// Matrix-core layouts (A [32 x 2], B [2 x 32], C [32 x 32] per instruction; lane l, half hl = l / 32):
+//   S^T = K Q^T : A = keys (row l % 32), B = queries (column l % 32); the two operands read the SAME coordinates in
+//                 the same order, so any order of the reduction is right: each lane reads runs of 16.
+//   C element r of lane l is key 8 (r / 4) + 4 hl + r % 4, query l % 32: a lane owns ONE query and 16 of the 32 keys,
+//                 its partner lane l ^ 32 the other 16.
+//   O^T = V^T P^T: A = values (channel l % 32 of key (r, hl)), B = the lane's own weights p[r]: no shuffle between
+//                 the two products.  C element r is channel 8 (r / 4) + 4 hl + r % 4 of the lane's query.
+#include "mixers_common.cuh"
+
+namespace swm {
+
+using f32x16 = __attribute__((ext_vector_type(16))) float;
+
+constexpr int kQT = 32;               // query rows and keys per tile
+
+// 16 consecutive coordinates [c0, c0 + 16) of a row of `size` coordinates, zeros beyond; `vec`: size % 8 == 0
+template <typename T>
+__device__ __forceinline__ void load_run16(float (&out)[16], const void* base, int64_t row_off, int c0, int size,
+                                           bool row_ok, bool vec);
+template <>
+__device__ __forceinline__ void load_run16<float>(float (&out)[16], const void* base, int64_t row_off, int c0,
+                                                  int size, bool row_ok, bool vec) {
+  const float* p = static_cast<const float*>(base) + row_off;
+  if (vec) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (row_ok && c0 + 4 * j + 4 <= size) v = *reinterpret_cast<const float4*>(p + c0 + 4 * j);
+      out[4 * j] = v.x; out[4 * j + 1] = v.y; out[4 * j + 2] = v.z; out[4 * j + 3] = v.w;
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 16; ++j) out[j] = (row_ok && c0 + j < size) ? p[c0 + j] : 0.0f;
+  }
+}
+template <>
+__device__ __forceinline__ void load_run16<bf16_t>(float (&out)[16], const void* base, int64_t row_off, int c0,
+                                                   int size, bool row_ok, bool vec) {
+  const uint16_t* p = static_cast<const uint16_t*>(base) + row_off;
+  if (vec) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      uint4 v = make_uint4(0u, 0u, 0u, 0u);
+      if (row_ok && c0 + 8 * j + 8 <= size) v = *reinterpret_cast<const uint4*>(p + c0 + 8 * j);
+      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        out[8 * j + 2 * e] = __uint_as_float(w[e] << 16);
+        out[8 * j + 2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 16; ++j) out[j] = (row_ok && c0 + j < size) ? sw::bf16_bits_to_float(p[c0 + j]) : 0.0f;
+  }
+}
+
+// -> sequence and first new token of tile `tile` when every sequence's new tokens are cut into runs of `tpt`;
+//    returns the tokens in the tile (0: no such tile)
+__device__ __forceinline__ int find_query_tile(const int32_t* __restrict__ q_start, int num_seqs, int tile, int tpt,
+                                               int* seq, int* tok0) {
+  for (int s = 0; s < num_seqs; ++s) {
+    const int n = q_start[s + 1] - q_start[s];
+    const int tiles = (n + tpt - 1) / tpt;
+    if (tile < tiles) {
+      *seq = s;
+      *tok0 = tile * tpt;
+      return min(tpt, n - tile * tpt);
+    }
+    tile -= tiles;
+  }
+  return 0;
+}
+
+// NVB: 32-channel blocks of the value size
+template <typename T, int NVB>
+__global__ __launch_bounds__(256) void capped_attention_kernel(
+    void* __restrict__ out, const float* __restrict__ q, const void* __restrict__ key_cache,
+    const void* __restrict__ value_cache, const void* __restrict__ gate, int64_t gate_stride,
+    const int32_t* __restrict__ block_tables, int table_width, const int32_t* __restrict__ q_start,
+    const int32_t* __restrict__ ctx_len, int num_seqs, int heads, int kv_heads, int dim, int vdim, int page_size,
+    float scale, float softcap, int window, int tpt) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  const int R = heads / kv_heads;
+  const int dblocks = (dim + 31) / 32;
+  const int qstride = dblocks * 32 + 4;
+  const int nw = blockDim.x >> 6;
+  const int ostride = NVB * 32 + 1;
+  float* Qs = lds;                                           // [32][qstride], scaled queries, zero padded
+  float* Ml = Qs + kQT * qstride;                            // [nw][32][2]: running maximum and sum
+  float* Os = Ml + nw * kQT * 2;                             // [nw][32][ostride]
+
+  int seq, tok0;
+  const int ntok = find_query_tile(q_start, num_seqs, blockIdx.x, tpt, &seq, &tok0);
+  if (ntok == 0) return;                                     // uniform over the workgroup
+  const int g = blockIdx.y;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int qi = lane & 31, hl = lane >> 5;
+  const int64_t row0 = q_start[seq] + tok0;
+  const int ctx = ctx_len[seq];
+  const int32_t* table = block_tables + (int64_t)seq * table_width;
+
+  for (int e = threadIdx.x; e < kQT * dblocks * 32; e += blockDim.x) {
+    const int r = e / (dblocks * 32), c = e % (dblocks * 32);
+    const int tt = r / R, hh = r % R;
+    float v = 0.0f;
+    if (tt < ntok && c < dim) v = q[(row0 + tt) * (int64_t)heads * dim + (int64_t)(g * R + hh) * dim + c] * scale;
+    Qs[r * qstride + c] = v;
+  }
+  __syncthreads();
+
+  const int first_pos = ctx + tok0, last_pos = ctx + tok0 + ntok - 1;
+  // rows without a token behave like the tile's last token and are never stored
+  const int pos_q = first_pos + min(qi / R, ntok - 1);
+  // keys below every row's window are skipped as whole tiles
+  const int lowest = window > 0 ? max(0, first_pos - window + 1) : 0;
+  const int tile_lo = lowest / kQT, tile_hi = last_pos / kQT;
+  const bool kvec = dim % 8 == 0;
+
+  f32x16 o[NVB];
+#pragma unroll
+  for (int b = 0; b < NVB; ++b)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[b][r] = 0.0f;
+  float m_run = -INFINITY, l_run = 0.0f;
+
+  for (int kt = tile_lo + wave; kt <= tile_hi; kt += nw) {
+    const int k0 = kt * kQT;
+    // ---- S^T = K Q^T
+    const int key = k0 + qi;
+    const bool key_ok = key <= last_pos;
+    int64_t krow = 0;
+    if (key_ok) krow = ((int64_t)table[key / page_size] * page_size + key % page_size) * kv_heads + g;
+    f32x16 s;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s[r] = 0.0f;
+    for (int db = 0; db < dblocks; ++db) {
+      const int c0 = db * 32 + hl * 16;
+      float kf[16];
+      load_run16<T>(kf, key_cache, krow * dim, c0, dim, key_ok, kvec);
+      const float4* qp = reinterpret_cast<const float4*>(Qs + qi * qstride + c0);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float4 qv = qp[j];
+        s = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[4 * j], qv.x, s, 0, 0, 0);
+        s = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[4 * j + 1], qv.y, s, 0, 0, 0);
+        s = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[4 * j + 2], qv.z, s, 0, 0, 0);
+        s = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[4 * j + 3], qv.w, s, 0, 0, 0);
+      }
+    }
+    // ---- cap, mask, running softmax (this lane: query qi, keys (r, hl))
+    float p[16];
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int kj = k0 + 8 * (r / 4) + 4 * hl + (r % 4);
+      float v = s[r];
+      if (softcap > 0.0f) v = softcap * tanhf(v / softcap);
+      const bool seen = kj <= pos_q && (window <= 0 || pos_q - kj < window);
+      v = seen ? v : -INFINITY;
+      p[r] = v;
+      tmax = fmaxf(tmax, v);
+    }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float m_new = fmaxf(m_run, tmax);
+    const float m_use = m_new == -INFINITY ? 0.0f : m_new;
+    const float alpha = expf(m_run - m_use);                 // 0 while nothing has been seen
+    float psum = 0.0f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      p[r] = expf(p[r] - m_use);
+      psum += p[r];
+    }
+    psum += __shfl_xor(psum, 32, 64);
+    l_run = l_run * alpha + psum;
+    m_run = m_new;
+    // ---- O^T = alpha O^T + V^T P^T
+    int64_t vrow[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int kj = k0 + 8 * (r / 4) + 4 * hl + (r % 4);
+      vrow[r] = kj <= last_pos ? ((int64_t)table[kj / page_size] * page_size + kj % page_size) * kv_heads + g : -1;
+    }
+#pragma unroll
+    for (int b = 0; b < NVB; ++b) {
+      const int vc = b * 32 + qi;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[b][r] *= alpha;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        float vv = 0.0f;
+        if (vc < vdim && vrow[r] >= 0) vv = ld<T>(value_cache, vrow[r] * vdim + vc);
+        o[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv, p[r], o[b], 0, 0, 0);
+      }
+    }
+  }
+
+  // ---- join the waves
+  if (hl == 0) {
+    Ml[(wave * kQT + qi) * 2] = m_run;
+    Ml[(wave * kQT + qi) * 2 + 1] = l_run;
+  }
+#pragma unroll
+  for (int b = 0; b < NVB; ++b)
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+      Os[(wave * kQT + qi) * ostride + b * 32 + 8 * (r / 4) + 4 * hl + (r % 4)] = o[b][r];
+  __syncthreads();
+  for (int e = threadIdx.x; e < kQT * vdim; e += blockDim.x) {
+    const int r = e / vdim, c = e % vdim;
+    const int tt = r / R, hh = r % R;
+    if (tt >= ntok) continue;
+    float m_all = -INFINITY;
+    for (int w = 0; w < nw; ++w) m_all = fmaxf(m_all, Ml[(w * kQT + r) * 2]);
+    float num = 0.0f, den = 0.0f;
+    for (int w = 0; w < nw; ++w) {
+      const float f = expf(Ml[(w * kQT + r) * 2] - m_all);  // a wave that saw no key: exp(-inf) = 0
+      den += f * Ml[(w * kQT + r) * 2 + 1];
+      num += f * Os[(w * kQT + r) * ostride + c];
+    }
+    float v = num / den;
+    const int64_t col = (int64_t)(g * R + hh) * vdim + c;
+    if (gate != nullptr) v *= sigmoidf_(ld<T>(gate, (row0 + tt) * gate_stride + col));
+    st<T>(out, (row0 + tt) * (int64_t)heads * vdim + col, v);
+  }
+}
+
+template <typename T, int NVB>
+int launch_capped_attention(void* out, const float* q, const void* key_cache, const void* value_cache, const void* gate,
+                            int64_t gate_stride, const int32_t* block_tables, int table_width, const int32_t* q_start,
+                            const int32_t* ctx_len, int64_t rows, int num_seqs, int heads, int kv_heads, int dim,
+                            int vdim, int page_size, float scale, float softcap, int window, hipStream_t stream) {
+  const int R = heads / kv_heads;
+  const int tpt = kQT / R;
+  const int dblocks = (dim + 31) / 32;
+  auto lds_bytes = [&](int nw) {
+    return (size_t)(kQT * (dblocks * 32 + 4) + nw * kQT * 2 + nw * kQT * (NVB * 32 + 1)) * sizeof(float);
+  };
+  int nw = 4;
+  while (nw > 1 && lds_bytes(nw) > 150 * 1024) nw >>= 1;
+  SW_CHECK_ARG(lds_bytes(nw) <= 160 * 1024, "capped_attention: key size %d with value size %d needs too much LDS", dim,
+               vdim);
+  auto kernel = capped_attention_kernel<T, NVB>;
+  static size_t allowed = 0;                                 // per instantiation
+  if (lds_bytes(nw) > allowed) {
+    SW_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     (int)lds_bytes(nw)));
+    allowed = lds_bytes(nw);
+  }
+  const dim3 grid((unsigned)((rows + tpt - 1) / tpt + num_seqs), (unsigned)kv_heads);
+  hipLaunchKernelGGL(kernel, grid, dim3(64 * nw), lds_bytes(nw), stream, out, q, key_cache, value_cache, gate,
+                     gate_stride, block_tables, table_width, q_start, ctx_len, num_seqs, heads, kv_heads, dim, vdim,
+                     page_size, scale, softcap, window, tpt);
+  SW_CHECK_LAUNCH();
+  return SW_OK;
+}
+
+}  // namespace swm
+
+extern "C" int swm_capped_attention(void* out, const float* q, const void* key_cache, const void* value_cache,
+                                    const void* gate, int64_t gate_stride, const int32_t* block_tables,
+                                    int table_width, const int32_t* q_start, const int32_t* ctx_len, int64_t rows,
+                                    int num_seqs, int heads, int kv_heads, int dim, int vdim, int page_size,
+                                    float scale, float softcap, int window, int act_dtype, void* stream) {
+  using namespace swm;
+  if (rows == 0 || num_seqs == 0) return SW_OK;
+  SW_CHECK_ARG(act_ok(act_dtype), "capped_attention: unsupported dtype %d", act_dtype);
+  SW_CHECK_ARG(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && heads / kv_heads <= kQT,
+               "capped_attention: %d query heads on %d key/value heads (at most %d per key/value head)", heads, kv_heads,
+               kQT);
+  SW_CHECK_ARG(dim > 0 && vdim > 0 && vdim <= 256 && page_size > 0 && table_width > 0 && rows < (1ll << 31),
+               "capped_attention: key size %d, value size %d (at most 256)", dim, vdim);
+  const int nvb = (vdim + 31) / 32;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+#define SWM_CAPPED_CASE(N)                                                                                              \
+  case N:                                                                                                               \
+    SWM_DISPATCH_ACT(act_dtype, return (launch_capped_attention<T, N>(                                                  \
+                                    out, q, key_cache, value_cache, gate, gate_stride, block_tables, table_width,       \
+                                    q_start, ctx_len, rows, num_seqs, heads, kv_heads, dim, vdim, page_size, scale,     \
+                                    softcap, window, s)););                                                             \
+    break;
+  switch (nvb) {
+    SWM_CAPPED_CASE(1)
+    SWM_CAPPED_CASE(2)
+    SWM_CAPPED_CASE(3)
+    SWM_CAPPED_CASE(4)
+    SWM_CAPPED_CASE(5)
+    SWM_CAPPED_CASE(6)
+    SWM_CAPPED_CASE(7)
+    SWM_CAPPED_CASE(8)
+  }
+#undef SWM_CAPPED_CASE
+  return SW_OK;
+}

@@ -13,6 +13,14 @@ namespace swm {
 constexpr int TM = 32, TN = 64, TK = 32, kFfnThreads = 256;
 
 __device__ __forceinline__ float gelu_erf(float z) { return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f)); }
+// activation of an expert's hidden layer: SWM_ACT_GELU (exact gelu) or SWM_ACT_RELU2 (the square of relu)
+__device__ __forceinline__ float expert_act(float z, int activation) {
+  if (activation == SWM_ACT_RELU2) {
+    const float r = fmaxf(z, 0.0f);
+    return r * r;
+  }
+  return gelu_erf(z);
+}
 
 // -> expert and first sorted row of this workgroup's tile of `tm` rows, rows in it (0: nothing to do)
 __device__ __forceinline__ int find_tile(const int32_t* __restrict__ expert_start, int num_experts, int tile,
@@ -76,7 +84,7 @@ template <typename T>
 __global__ __launch_bounds__(kFfnThreads) void expert_up_gelu_kernel(
     void* __restrict__ hidden, const void* __restrict__ x, const void* __restrict__ up,
     const int32_t* __restrict__ order, const int32_t* __restrict__ expert_start, int num_experts, int width, int ff,
-    int top) {
+    int top, int activation) {
   __shared__ float As[TM][TK + 1];
   __shared__ float Bs[TN][TK + 1];
   int e, row0;
@@ -94,7 +102,7 @@ __global__ __launch_bounds__(kFfnThreads) void expert_up_gelu_kernel(
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int n = n0 + tx + 16 * j;
-      if (n < ff) st<T>(hidden, (int64_t)(row0 + r) * ff + n, gelu_erf(acc[i][j]));
+      if (n < ff) st<T>(hidden, (int64_t)(row0 + r) * ff + n, expert_act(acc[i][j], activation));
     }
   }
 }
@@ -103,7 +111,7 @@ template <typename T>
 __global__ __launch_bounds__(kFfnThreads) void expert_down_kernel(
     float* __restrict__ out, const void* __restrict__ hidden, const void* __restrict__ down,
     const int32_t* __restrict__ order, const int32_t* __restrict__ expert_start, int num_experts, int width, int ff,
-    int top, float weight) {
+    int top, float weight, const float* __restrict__ pair_weight) {
   __shared__ float As[TM][TK + 1];
   __shared__ float Bs[TN][TK + 1];
   int e, row0;
@@ -118,14 +126,16 @@ __global__ __launch_bounds__(kFfnThreads) void expert_down_kernel(
   for (int i = 0; i < 2; ++i) {
     const int r = 2 * ty + i;
     if (r >= rows) continue;
-    const int64_t dst = order[row0 + r] / top;
+    const int pair = order[row0 + r];
+    const int64_t dst = pair / top;
+    const float wt = pair_weight != nullptr ? weight * pair_weight[pair] : weight;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int n = n0 + tx + 16 * j;
       if (n >= width) continue;
       float* p = out + dst * width + n;
-      if (top == 1) *p += weight * acc[i][j];           // a row has one expert: nobody else writes it
-      else atomicAdd(p, weight * acc[i][j]);
+      if (top == 1) *p += wt * acc[i][j];               // a row has one expert: nobody else writes it
+      else atomicAdd(p, wt * acc[i][j]);
     }
   }
 }
@@ -182,7 +192,7 @@ __device__ __forceinline__ void for_each_acc(const f32x16& acc, F&& f) {
 __global__ __launch_bounds__(kFfnThreads) void expert_up_gelu_mfma_kernel(
     uint16_t* __restrict__ hidden, const uint16_t* __restrict__ x, const uint16_t* __restrict__ up,
     const int32_t* __restrict__ order, const int32_t* __restrict__ expert_start, int num_experts, int width, int ff,
-    int top) {
+    int top, int activation) {
   __shared__ __attribute__((aligned(16))) uint16_t As[MM][MK + MPAD];
   __shared__ __attribute__((aligned(16))) uint16_t Bs[MN][MK + MPAD];
   int e, row0;
@@ -193,14 +203,14 @@ __global__ __launch_bounds__(kFfnThreads) void expert_up_gelu_mfma_kernel(
   tile_gemm_mfma(acc, x, [&](int r) { return (int64_t)(order[row0 + r] / top); }, rows, up, (int64_t)e * ff * width, n0,
                  ff, width, As, Bs);
   for_each_acc(acc, [&](int r, int c, float v) {
-    if (r < rows && n0 + c < ff) hidden[(int64_t)(row0 + r) * ff + n0 + c] = sw::float_to_bf16_bits(gelu_erf(v));
+    if (r < rows && n0 + c < ff) hidden[(int64_t)(row0 + r) * ff + n0 + c] = sw::float_to_bf16_bits(expert_act(v, activation));
   });
 }
 
 __global__ __launch_bounds__(kFfnThreads) void expert_down_mfma_kernel(
     float* __restrict__ out, const uint16_t* __restrict__ hidden, const uint16_t* __restrict__ down,
     const int32_t* __restrict__ order, const int32_t* __restrict__ expert_start, int num_experts, int width, int ff,
-    int top, float weight) {
+    int top, float weight, const float* __restrict__ pair_weight) {
   __shared__ __attribute__((aligned(16))) uint16_t As[MM][MK + MPAD];
   __shared__ __attribute__((aligned(16))) uint16_t Bs[MN][MK + MPAD];
   int e, row0;
@@ -212,9 +222,11 @@ __global__ __launch_bounds__(kFfnThreads) void expert_down_mfma_kernel(
                  ff, As, Bs);
   for_each_acc(acc, [&](int r, int c, float v) {
     if (r < rows && n0 + c < width) {
-      float* p = out + (int64_t)(order[row0 + r] / top) * width + n0 + c;
-      if (top == 1) *p += weight * v;
-      else atomicAdd(p, weight * v);
+      const int pair = order[row0 + r];
+      const float wt = pair_weight != nullptr ? weight * pair_weight[pair] : weight;
+      float* p = out + (int64_t)(pair / top) * width + n0 + c;
+      if (top == 1) *p += wt * v;
+      else atomicAdd(p, wt * v);
     }
   });
 }
@@ -226,22 +238,30 @@ extern "C" {
 int swm_expert_up_gelu(void* hidden, const void* x, const void* up, const int32_t* order,
                        const int32_t* expert_start, int num_experts, int64_t sorted_rows, int width, int ff,
                        int top, int act_dtype, void* stream) {
+  return swm_expert_up(hidden, x, up, order, expert_start, num_experts, sorted_rows, width, ff, top, SWM_ACT_GELU,
+                       act_dtype, stream);
+}
+
+int swm_expert_up(void* hidden, const void* x, const void* up, const int32_t* order, const int32_t* expert_start,
+                  int num_experts, int64_t sorted_rows, int width, int ff, int top, int activation, int act_dtype,
+                  void* stream) {
   using namespace swm;
   if (sorted_rows == 0) return SW_OK;
+  SW_CHECK_ARG(activation == SWM_ACT_GELU || activation == SWM_ACT_RELU2, "expert_up: unknown activation %d", activation);
   SW_CHECK_ARG(act_ok(act_dtype), "expert_up_gelu: unsupported dtype %d", act_dtype);
   SW_CHECK_ARG(num_experts > 0 && width > 0 && ff > 0 && top > 0 && sorted_rows < (1ll << 30), "expert_up_gelu: bad shape");
   if (act_dtype == SW_BF16 && width % 8 == 0) {
     const dim3 mgrid((unsigned)((sorted_rows + MM - 1) / MM + num_experts), (unsigned)((ff + MN - 1) / MN));
     hipLaunchKernelGGL(expert_up_gelu_mfma_kernel, mgrid, dim3(kFfnThreads), 0, static_cast<hipStream_t>(stream),
                        static_cast<uint16_t*>(hidden), static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(up),
-                       order, expert_start, num_experts, width, ff, top);
+                       order, expert_start, num_experts, width, ff, top, activation);
     SW_CHECK_LAUNCH();
     return SW_OK;
   }
   const dim3 grid((unsigned)((sorted_rows + TM - 1) / TM + num_experts), (unsigned)((ff + TN - 1) / TN));
   SWM_DISPATCH_ACT(act_dtype, hipLaunchKernelGGL(expert_up_gelu_kernel<T>, grid, dim3(kFfnThreads), 0,
                                                  static_cast<hipStream_t>(stream), hidden, x, up, order, expert_start,
-                                                 num_experts, width, ff, top););
+                                                 num_experts, width, ff, top, activation););
   SW_CHECK_LAUNCH();
   return SW_OK;
 }
@@ -249,6 +269,13 @@ int swm_expert_up_gelu(void* hidden, const void* x, const void* up, const int32_
 int swm_expert_down(float* out, const void* hidden, const void* down, const int32_t* order,
                     const int32_t* expert_start, int num_experts, int64_t sorted_rows, int width, int ff,
                     int top, float weight, int act_dtype, void* stream) {
+  return swm_expert_down_weighted(out, hidden, down, order, expert_start, num_experts, sorted_rows, width, ff, top,
+                                  weight, nullptr, act_dtype, stream);
+}
+
+int swm_expert_down_weighted(float* out, const void* hidden, const void* down, const int32_t* order,
+                             const int32_t* expert_start, int num_experts, int64_t sorted_rows, int width, int ff,
+                             int top, float weight, const float* pair_weight, int act_dtype, void* stream) {
   using namespace swm;
   if (sorted_rows == 0) return SW_OK;
   SW_CHECK_ARG(act_ok(act_dtype), "expert_down: unsupported dtype %d", act_dtype);
@@ -257,14 +284,14 @@ int swm_expert_down(float* out, const void* hidden, const void* down, const int3
     const dim3 mgrid((unsigned)((sorted_rows + MM - 1) / MM + num_experts), (unsigned)((width + MN - 1) / MN));
     hipLaunchKernelGGL(expert_down_mfma_kernel, mgrid, dim3(kFfnThreads), 0, static_cast<hipStream_t>(stream), out,
                        static_cast<const uint16_t*>(hidden), static_cast<const uint16_t*>(down), order, expert_start,
-                       num_experts, width, ff, top, weight);
+                       num_experts, width, ff, top, weight, pair_weight);
     SW_CHECK_LAUNCH();
     return SW_OK;
   }
   const dim3 grid((unsigned)((sorted_rows + TM - 1) / TM + num_experts), (unsigned)((width + TN - 1) / TN));
   SWM_DISPATCH_ACT(act_dtype, hipLaunchKernelGGL(expert_down_kernel<T>, grid, dim3(kFfnThreads), 0,
                                                  static_cast<hipStream_t>(stream), out, hidden, down, order,
-                                                 expert_start, num_experts, width, ff, top, weight););
+                                                 expert_start, num_experts, width, ff, top, weight, pair_weight););
   SW_CHECK_LAUNCH();
   return SW_OK;
 }

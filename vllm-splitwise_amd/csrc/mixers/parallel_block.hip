@@ -1,0 +1,268 @@
+// Pieces of a decoder layer whose two sublayers read ONE norm of an fp32 residual stream:
+//   * stream_add_norm: the sublayers' outputs are summed into the stream and the next layer's norm (per-channel
+//     weight with an offset, so that a weight stored around zero is offset + w) is taken in the same pass;
+//   * clamped_glu / relu2: activations between the library GEMMs of a feed-forward;
+//   * rope_cache: partial rotary embedding on neighbouring pairs from a table of per-pair frequencies (angles
+//     from fp32 positions), rotated queries out in fp32, rotated keys and values into the paged cache;
+//   * group_router: sigmoid router with a selection bias, a limit to the best groups of experts and weights
+//     normalised over the chosen ones.
+// All arithmetic is fp32; activations are read and written in the model's dtype.
+#include "mixers_common.cuh"
+
+namespace swm {
+
+constexpr int kPbThreads = 256;
+
+// residual += (a + b + c);  out = residual / sqrt(mean(residual^2) + eps) * (offset + weight)
+template <typename T>
+__global__ __launch_bounds__(kPbThreads) void stream_add_norm_kernel(
+    float* __restrict__ residual, const void* __restrict__ a, int64_t a_stride, const void* __restrict__ b,
+    int64_t b_stride, const float* __restrict__ c, const float* __restrict__ weight, float offset, float eps,
+    void* __restrict__ out, int width) {
+  __shared__ float red[16];
+  const int64_t t = blockIdx.x;
+  float* r = residual + t * (int64_t)width;
+  float ss = 0.0f;
+  for (int i = threadIdx.x; i < width; i += kPbThreads) {
+    float v = r[i];
+    if (a != nullptr || b != nullptr || c != nullptr) {
+      float add = 0.0f;
+      if (a != nullptr) add += ld<T>(a, t * a_stride + i);
+      if (b != nullptr) add += ld<T>(b, t * b_stride + i);
+      if (c != nullptr) add += c[t * (int64_t)width + i];
+      v += add;
+      r[i] = v;
+    }
+    ss += v * v;
+  }
+  if (out == nullptr) return;
+  ss = block_sum(ss, red);
+  const float f = 1.0f / sqrtf(ss / (float)width + eps);
+  for (int i = threadIdx.x; i < width; i += kPbThreads)
+    st<T>(out, t * (int64_t)width + i, r[i] * f * (offset + weight[i]));
+}
+
+// in [rows, 2 * ff] (gate | up):  g = min(gate, limit), u = clamp(up, -limit, limit);  out = g sigmoid(alpha g) (u + shift)
+template <typename T>
+__global__ __launch_bounds__(kPbThreads) void clamped_glu_kernel(void* __restrict__ out, const void* __restrict__ in,
+                                                                 int64_t in_stride, int ff, float alpha, float limit,
+                                                                 float shift) {
+  const int64_t t = blockIdx.x;
+  for (int i = blockIdx.y * kPbThreads + threadIdx.x; i < ff; i += gridDim.y * kPbThreads) {
+    const float g = fminf(ld<T>(in, t * in_stride + i), limit);
+    const float u = fminf(fmaxf(ld<T>(in, t * in_stride + ff + i), -limit), limit);
+    st<T>(out, t * (int64_t)ff + i, g * sigmoidf_(alpha * g) * (u + shift));
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kPbThreads) void relu2_kernel(void* __restrict__ out, const void* __restrict__ in,
+                                                           int64_t in_stride, int ff) {
+  const int64_t t = blockIdx.x;
+  for (int i = blockIdx.y * kPbThreads + threadIdx.x; i < ff; i += gridDim.y * kPbThreads) {
+    const float z = fmaxf(ld<T>(in, t * in_stride + i), 0.0f);
+    st<T>(out, t * (int64_t)ff + i, z * z);
+  }
+}
+
+// one workgroup per row; a thread per (head, pair) or per passed-through coordinate
+template <typename T>
+__global__ __launch_bounds__(kPbThreads) void rope_cache_kernel(
+    float* __restrict__ q_out, const void* __restrict__ q, const void* __restrict__ k, const void* __restrict__ v,
+    int64_t in_stride, const int64_t* __restrict__ positions, const float* __restrict__ inv_freq, int rot_dims,
+    void* __restrict__ key_cache, void* __restrict__ value_cache, const int64_t* __restrict__ slot_mapping, int heads,
+    int kv_heads, int dim, int vdim) {
+  const int64_t t = blockIdx.x;
+  const int64_t row = t * in_stride;
+  const float pos = (float)positions[t];
+  const int half = rot_dims / 2, pairs = dim / 2;          // pairs beyond `half` pass through; so does an odd last one
+  // queries
+  for (int e = threadIdx.x; e < heads * pairs; e += kPbThreads) {
+    const int h = e / pairs, i = e % pairs;
+    const int64_t src = row + h * dim + 2 * i, dst = t * (int64_t)heads * dim + h * dim + 2 * i;
+    const float a = ld<T>(q, src), b = ld<T>(q, src + 1);
+    if (i < half) {
+      float s, c;
+      sincosf(pos * inv_freq[i], &s, &c);
+      q_out[dst] = a * c - b * s;
+      q_out[dst + 1] = b * c + a * s;
+    } else {
+      q_out[dst] = a;
+      q_out[dst + 1] = b;
+    }
+  }
+  if (dim & 1)
+    for (int h = threadIdx.x; h < heads; h += kPbThreads)
+      q_out[t * (int64_t)heads * dim + h * dim + dim - 1] = ld<T>(q, row + h * dim + dim - 1);
+  if (k == nullptr) return;
+  const int64_t slot = slot_mapping[t];
+  if (slot < 0) return;
+  for (int e = threadIdx.x; e < kv_heads * pairs; e += kPbThreads) {
+    const int h = e / pairs, i = e % pairs;
+    const int64_t src = row + h * dim + 2 * i, dst = slot * (int64_t)kv_heads * dim + h * dim + 2 * i;
+    const float a = ld<T>(k, src), b = ld<T>(k, src + 1);
+    if (i < half) {
+      float s, c;
+      sincosf(pos * inv_freq[i], &s, &c);
+      st<T>(key_cache, dst, a * c - b * s);
+      st<T>(key_cache, dst + 1, b * c + a * s);
+    } else {
+      st<T>(key_cache, dst, a);
+      st<T>(key_cache, dst + 1, b);
+    }
+  }
+  if (dim & 1)
+    for (int h = threadIdx.x; h < kv_heads; h += kPbThreads)
+      st<T>(key_cache, slot * (int64_t)kv_heads * dim + h * dim + dim - 1, ld<T>(k, row + h * dim + dim - 1));
+  for (int e = threadIdx.x; e < kv_heads * vdim; e += kPbThreads)
+    st<T>(value_cache, slot * (int64_t)kv_heads * vdim + e, ld<T>(v, row + e));
+}
+
+// one wave per row: the router's products over the lanes, the choice by lane 0
+constexpr int kMaxRouterExperts = 256;
+
+template <typename T>
+__global__ __launch_bounds__(256) void group_router_kernel(
+    int32_t* __restrict__ chosen, float* __restrict__ weights, const void* __restrict__ h, int64_t h_stride,
+    const float* __restrict__ router, const float* __restrict__ correction, int64_t rows, int width, int experts,
+    int top, int groups, int keep, float scale) {
+  __shared__ float s_score[4][kMaxRouterExperts];
+  __shared__ float s_choice[4][kMaxRouterExperts];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int64_t t = (int64_t)blockIdx.x * 4 + wave;
+  if (t >= rows) return;                                   // uniform over the wave; no workgroup barrier below
+  float* score = s_score[wave];
+  float* choice = s_choice[wave];
+  for (int e = 0; e < experts; ++e) {
+    float z = 0.0f;
+    for (int i = lane; i < width; i += 64) z += router[(int64_t)e * width + i] * ld<T>(h, t * h_stride + i);
+    z = sw::wave_sum(z);
+    if (lane == 0) {
+      const float s = sigmoidf_(z);
+      score[e] = s;
+      choice[e] = s + (correction != nullptr ? correction[e] : 0.0f);
+    }
+  }
+  if (lane != 0) return;
+  const float kOut = -INFINITY;
+  if (groups > 1 && keep < groups) {
+    const int size = experts / groups;
+    // a group's score: its two largest choice scores; the groups outside the best `keep` leave the choice
+    uint64_t dropped[kMaxRouterExperts / 64] = {};
+    for (int drop = 0; drop < groups - keep; ++drop) {
+      int worst = -1;
+      float worst_score = 0.0f;
+      for (int g = groups - 1; g >= 0; --g) {                // ties: the later group goes first
+        if ((dropped[g >> 6] >> (g & 63)) & 1ull) continue;
+        float first = kOut, second = kOut;
+        for (int j = 0; j < size; ++j) {
+          const float c = choice[g * size + j];
+          if (c > first) { second = first; first = c; }
+          else if (c > second) second = c;
+        }
+        const float gs = size > 1 ? first + second : first;
+        if (worst < 0 || gs < worst_score) { worst = g; worst_score = gs; }
+      }
+      dropped[worst >> 6] |= 1ull << (worst & 63);
+      for (int j = 0; j < size; ++j) choice[worst * size + j] = kOut;
+    }
+  }
+  float total = 0.0f;
+  for (int n = 0; n < top; ++n) {
+    int best = 0;
+    float best_choice = choice[0];
+    for (int e = 1; e < experts; ++e)
+      if (choice[e] > best_choice) { best = e; best_choice = choice[e]; }   // ties: the earlier expert
+    choice[best] = kOut;                                    // (an expert already taken has -inf and loses every tie but the last)
+    chosen[t * top + n] = best;
+    weights[t * top + n] = score[best];
+    total += score[best];
+  }
+  const float f = scale / (total + 1e-20f);
+  for (int n = 0; n < top; ++n) weights[t * top + n] *= f;
+}
+
+}  // namespace swm
+
+extern "C" {
+
+int swm_stream_add_norm(float* residual, const void* a, int64_t a_stride, const void* b, int64_t b_stride,
+                        const float* c, const float* weight, float offset, float eps, void* out, int64_t rows,
+                        int width, int act_dtype, void* stream) {
+  using namespace swm;
+  if (rows == 0) return SW_OK;
+  SW_CHECK_ARG(act_ok(act_dtype), "stream_add_norm: unsupported dtype %d", act_dtype);
+  SW_CHECK_ARG(width > 0 && rows < (1ll << 31) && (out == nullptr || weight != nullptr), "stream_add_norm: bad shape");
+  SWM_DISPATCH_ACT(act_dtype, hipLaunchKernelGGL(stream_add_norm_kernel<T>, dim3((unsigned)rows), dim3(kPbThreads), 0,
+                                                 static_cast<hipStream_t>(stream), residual, a, a_stride, b, b_stride, c,
+                                                 weight, offset, eps, out, width););
+  SW_CHECK_LAUNCH();
+  return SW_OK;
+}
+
+int swm_clamped_glu(void* out, const void* in, int64_t in_stride, int64_t rows, int ff, float alpha, float limit,
+                    float shift, int act_dtype, void* stream) {
+  using namespace swm;
+  if (rows == 0) return SW_OK;
+  SW_CHECK_ARG(act_ok(act_dtype), "clamped_glu: unsupported dtype %d", act_dtype);
+  SW_CHECK_ARG(ff > 0 && rows < (1ll << 31) && limit > 0.0f, "clamped_glu: bad shape or limit");
+  const dim3 grid((unsigned)rows, (unsigned)std::min(8, (ff + kPbThreads - 1) / kPbThreads));
+  SWM_DISPATCH_ACT(act_dtype, hipLaunchKernelGGL(clamped_glu_kernel<T>, grid, dim3(kPbThreads), 0,
+                                                 static_cast<hipStream_t>(stream), out, in, in_stride, ff, alpha, limit,
+                                                 shift););
+  SW_CHECK_LAUNCH();
+  return SW_OK;
+}
+
+int swm_relu2(void* out, const void* in, int64_t in_stride, int64_t rows, int ff, int act_dtype, void* stream) {
+  using namespace swm;
+  if (rows == 0) return SW_OK;
+  SW_CHECK_ARG(act_ok(act_dtype), "relu2: unsupported dtype %d", act_dtype);
+  SW_CHECK_ARG(ff > 0 && rows < (1ll << 31), "relu2: bad shape");
+  const dim3 grid((unsigned)rows, (unsigned)std::min(8, (ff + kPbThreads - 1) / kPbThreads));
+  SWM_DISPATCH_ACT(act_dtype, hipLaunchKernelGGL(relu2_kernel<T>, grid, dim3(kPbThreads), 0,
+                                                 static_cast<hipStream_t>(stream), out, in, in_stride, ff););
+  SW_CHECK_LAUNCH();
+  return SW_OK;
+}
+
+int swm_rope_cache(float* q_out, const void* q, const void* k, const void* v, int64_t in_stride,
+                   const int64_t* positions, const float* inv_freq, int rot_dims, void* key_cache, void* value_cache,
+                   const int64_t* slot_mapping, int64_t rows, int heads, int kv_heads, int dim, int vdim, int act_dtype,
+                   void* stream) {
+  using namespace swm;
+  if (rows == 0) return SW_OK;
+  SW_CHECK_ARG(act_ok(act_dtype), "rope_cache: unsupported dtype %d", act_dtype);
+  SW_CHECK_ARG(heads > 0 && dim > 0 && rot_dims >= 0 && rot_dims <= dim && rot_dims % 2 == 0 && rows < (1ll << 31),
+               "rope_cache: %d rotated coordinates of %d", rot_dims, dim);
+  SW_CHECK_ARG(rot_dims == 0 || inv_freq != nullptr, "rope_cache: no frequencies");
+  SW_CHECK_ARG(k == nullptr || (v != nullptr && key_cache != nullptr && value_cache != nullptr &&
+                                slot_mapping != nullptr && kv_heads > 0 && vdim > 0),
+               "rope_cache: keys need values, caches and slots");
+  SWM_DISPATCH_ACT(act_dtype, hipLaunchKernelGGL(rope_cache_kernel<T>, dim3((unsigned)rows), dim3(kPbThreads), 0,
+                                                 static_cast<hipStream_t>(stream), q_out, q, k, v, in_stride, positions,
+                                                 inv_freq, rot_dims, key_cache, value_cache, slot_mapping, heads,
+                                                 kv_heads, dim, vdim););
+  SW_CHECK_LAUNCH();
+  return SW_OK;
+}
+
+int swm_group_router(int32_t* chosen, float* weights, const void* h, int64_t h_stride, const float* router,
+                     const float* correction, int64_t rows, int width, int experts, int top, int groups, int keep,
+                     float scale, int act_dtype, void* stream) {
+  using namespace swm;
+  if (rows == 0) return SW_OK;
+  SW_CHECK_ARG(act_ok(act_dtype), "group_router: unsupported dtype %d", act_dtype);
+  SW_CHECK_ARG(experts > 0 && experts <= kMaxRouterExperts && top > 0 && top <= experts && width > 0,
+               "group_router: %d experts (1..%d supported), top %d", experts, kMaxRouterExperts, top);
+  SW_CHECK_ARG(groups >= 1 && keep >= 1 && keep <= groups && experts % groups == 0 &&
+                   (int64_t)keep * (experts / groups) >= top,
+               "group_router: %d groups, %d kept, %d experts, top %d", groups, keep, experts, top);
+  SWM_DISPATCH_ACT(act_dtype, hipLaunchKernelGGL(group_router_kernel<T>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
+                                                 static_cast<hipStream_t>(stream), chosen, weights, h, h_stride, router,
+                                                 correction, rows, width, experts, top, groups, keep, scale););
+  SW_CHECK_LAUNCH();
+  return SW_OK;
+}
+
+}  // extern "C"

@@ -18,7 +18,7 @@ import torch
 
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_PKG_DIR, "libsplitwise_mixers.so")
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 SW_F32, SW_BF16 = 0, 2
 _ACT = {torch.float32: SW_F32, torch.bfloat16: SW_BF16}
@@ -37,7 +37,17 @@ _SIGNATURES = {
     "swm_head_norm_gate": [_p, _p, _p, _l, _p, _i, _f, _l, _i, _i, _i, _p],
     "swm_expert_up_gelu": [_p, _p, _p, _p, _p, _i, _l, _i, _i, _i, _i, _p],
     "swm_expert_down": [_p, _p, _p, _p, _p, _i, _l, _i, _i, _i, _f, _i, _p],
+    "swm_expert_up": [_p, _p, _p, _p, _p, _i, _l, _i, _i, _i, _i, _i, _p],
+    "swm_expert_down_weighted": [_p, _p, _p, _p, _p, _i, _l, _i, _i, _i, _f, _p, _i, _p],
+    "swm_stream_add_norm": [_p, _p, _l, _p, _l, _p, _p, _f, _f, _p, _l, _i, _i, _p],
+    "swm_clamped_glu": [_p, _p, _l, _l, _i, _f, _f, _f, _i, _p],
+    "swm_relu2": [_p, _p, _l, _l, _i, _i, _p],
+    "swm_rope_cache": [_p, _p, _p, _p, _l, _p, _p, _i, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p],
+    "swm_group_router": [_p, _p, _p, _l, _p, _p, _l, _i, _i, _i, _i, _i, _f, _i, _p],
+    "swm_capped_attention": [_p, _p, _p, _p, _p, _l, _p, _i, _p, _p, _l, _i, _i, _i, _i, _i, _i, _f, _f, _i, _i, _p],
+    "swm_lightning": [_p, _p, _p, _p, _l, _p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p],
 }
+ACT_GELU, ACT_RELU2 = 0, 1
 
 _lib = None
 
@@ -321,10 +331,13 @@ def head_norm_gate(out: torch.Tensor, o: torch.Tensor, gate: torch.Tensor, weigh
 
 
 def expert_ffn(out: torch.Tensor, x: torch.Tensor, up: torch.Tensor, down: torch.Tensor, order: torch.Tensor,
-               expert_start: torch.Tensor, top: int, weight: float) -> None:
+               expert_start: torch.Tensor, top: int, weight: float, activation: int = ACT_GELU,
+               pair_weight: Optional[torch.Tensor] = None) -> None:
     """out (fp32 [rows, width], zeroed by the caller) += weight * sum over each row's experts of
-    down[e] gelu(up[e] x[row]); ``order`` / ``expert_start`` as ``TableRoutedExperts.route`` makes them."""
-    _dev(out, x, up, down, order, expert_start)
+    pair_weight[row, choice] * down[e] act(up[e] x[row]); ``order`` / ``expert_start``: the (row, choice) pairs
+    sorted by expert and every expert's first sorted pair; ``activation``: ACT_GELU (exact gelu) or ACT_RELU2;
+    ``pair_weight`` fp32 [rows, top] (None: all 1)."""
+    _dev(out, x, up, down, order, expert_start, pair_weight)
     _f32c(out, "out")
     rows, width = x.shape
     experts, ff = up.shape[0], up.shape[1]
@@ -333,18 +346,182 @@ def expert_ffn(out: torch.Tensor, x: torch.Tensor, up: torch.Tensor, down: torch
           and order.dtype == torch.int32 and order.numel() == rows * top and order.is_contiguous()
           and expert_start.dtype == torch.int32 and expert_start.numel() == experts + 1
           and expert_start.is_contiguous(), "expert_ffn: shapes")
+    if pair_weight is not None:
+        _f32c(pair_weight, "pair_weight")
+        _need(pair_weight.numel() == rows * top, "expert_ffn: one weight per (row, choice)")
     pairs = rows * top
     hidden = torch.empty(pairs, ff, dtype=x.dtype, device=x.device)
     with _on_device_of(x):
         lib = load_library()
-        _check(lib.swm_expert_up_gelu(hidden.data_ptr(), x.data_ptr(), up.data_ptr(), order.data_ptr(),
-                                      expert_start.data_ptr(), experts, pairs, width, ff, top, _act(x), _stream(x)))
-        _check(lib.swm_expert_down(out.data_ptr(), hidden.data_ptr(), down.data_ptr(), order.data_ptr(),
-                                   expert_start.data_ptr(), experts, pairs, width, ff, top, weight, _act(x),
-                                   _stream(x)))
+        _check(lib.swm_expert_up(hidden.data_ptr(), x.data_ptr(), up.data_ptr(), order.data_ptr(),
+                                 expert_start.data_ptr(), experts, pairs, width, ff, top, activation, _act(x),
+                                 _stream(x)))
+        _check(lib.swm_expert_down_weighted(out.data_ptr(), hidden.data_ptr(), down.data_ptr(), order.data_ptr(),
+                                            expert_start.data_ptr(), experts, pairs, width, ff, top, weight,
+                                            None if pair_weight is None else pair_weight.data_ptr(), _act(x),
+                                            _stream(x)))
 
 
-ops = SimpleNamespace(expert_ffn=expert_ffn, 
+def _opt_ptr(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def stream_add_norm(residual: torch.Tensor, weight: Optional[torch.Tensor], offset: float, eps: float,
+                    out: Optional[torch.Tensor], a: Optional[torch.Tensor] = None, b: Optional[torch.Tensor] = None,
+                    c: Optional[torch.Tensor] = None) -> None:
+    """residual (fp32, in place) += a + b + c (a, b: the activation dtype, 2-D views; c: fp32), then
+    out = residual / rms(residual) * (offset + weight) in out's dtype (``out`` None: only the sum)."""
+    _dev(residual, weight, out, a, b, c)
+    _f32c(residual, "residual")
+    rows, width = residual.shape
+    act = out if out is not None else (a if a is not None else b)
+    _need(act is not None or c is not None, "stream_add_norm: nothing to do")
+    for t in (a, b):
+        if t is not None:
+            _need(t.shape == residual.shape and t.dtype == act.dtype, "stream_add_norm: addend")
+    if c is not None:
+        _f32c(c, "c")
+        _need(c.shape == residual.shape, "stream_add_norm: fp32 addend")
+    if out is not None:
+        _f32c(weight, "weight")
+        _need(out.shape == residual.shape and out.is_contiguous() and weight.numel() == width, "stream_add_norm: out")
+    with _on_device_of(residual):
+        _check(load_library().swm_stream_add_norm(
+            residual.data_ptr(), _opt_ptr(a), 0 if a is None else _rows(a, "a"), _opt_ptr(b),
+            0 if b is None else _rows(b, "b"), _opt_ptr(c), _opt_ptr(weight), offset, eps, _opt_ptr(out), rows, width,
+            SW_F32 if act is None else _act(act), _stream(residual)))
+
+
+def clamped_glu(out: torch.Tensor, gate_up: torch.Tensor, alpha: float, limit: float, shift: float) -> None:
+    """gate_up [rows, 2 * ff] = gate | up -> out [rows, ff] = g sigmoid(alpha g) (u + shift) with g = min(gate, limit),
+    u = clamp(up, -limit, limit)."""
+    _dev(out, gate_up)
+    rows, ff = out.shape
+    _need(out.is_contiguous() and gate_up.shape == (rows, 2 * ff) and gate_up.dtype == out.dtype, "clamped_glu: shapes")
+    with _on_device_of(out):
+        _check(load_library().swm_clamped_glu(out.data_ptr(), gate_up.data_ptr(), _rows(gate_up, "gate_up"), rows, ff,
+                                              alpha, limit, shift, _act(out), _stream(out)))
+
+
+def relu2(out: torch.Tensor, x: torch.Tensor) -> None:
+    _dev(out, x)
+    _need(out.is_contiguous() and x.shape == out.shape and x.dtype == out.dtype and out.dim() == 2, "relu2: shapes")
+    with _on_device_of(out):
+        _check(load_library().swm_relu2(out.data_ptr(), x.data_ptr(), _rows(x, "x"), out.shape[0], out.shape[1],
+                                        _act(out), _stream(out)))
+
+
+def rope_cache(q_out: torch.Tensor, q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.Tensor],
+               positions: torch.Tensor, inv_freq: Optional[torch.Tensor], heads: int, kv_heads: int, dim: int, vdim: int,
+               key_cache: Optional[torch.Tensor], value_cache: Optional[torch.Tensor],
+               slot_mapping: Optional[torch.Tensor]) -> None:
+    """q, k, v: column ranges of ONE projection output.  q_out fp32 = rotated q; rotated k and v go to the caches
+    [pages, page, kv_heads * size] (k None: a layer that reads another layer's keys)."""
+    _dev(q_out, q, k, v, positions, inv_freq, key_cache, value_cache, slot_mapping)
+    _f32c(q_out, "q_out")
+    stride = _rows(q, "q")
+    rows = q.shape[0]
+    rot = 0
+    if inv_freq is not None and inv_freq.numel() > 0:
+        _f32c(inv_freq, "inv_freq")
+        rot = 2 * inv_freq.numel()
+    _need(q.shape[1] == heads * dim and q_out.shape == q.shape and rot <= dim, "rope_cache: query shapes")
+    _need(positions.dtype == torch.int64 and positions.numel() == rows and positions.is_contiguous(),
+          "rope_cache: positions must be int64 [rows]")
+    if k is not None:
+        _need(v is not None and key_cache is not None and value_cache is not None and slot_mapping is not None,
+              "rope_cache: keys need values, caches and slots")
+        _need(_rows(k, "k") == stride and _rows(v, "v") == stride and k.dtype == q.dtype and v.dtype == q.dtype
+              and k.shape == (rows, kv_heads * dim) and v.shape == (rows, kv_heads * vdim),
+              "rope_cache: q, k, v must share rows and stride")
+        _need(key_cache.dtype == q.dtype and value_cache.dtype == q.dtype and key_cache.is_contiguous()
+              and value_cache.is_contiguous() and key_cache.shape[-1] == kv_heads * dim
+              and value_cache.shape[-1] == kv_heads * vdim
+              and key_cache.shape[0] * key_cache.shape[1] == value_cache.shape[0] * value_cache.shape[1],
+              "rope_cache: cache shapes")
+        _need(slot_mapping.dtype == torch.int64 and slot_mapping.numel() == rows and slot_mapping.is_contiguous(),
+              "rope_cache: slot_mapping must be int64 [rows]")
+    with _on_device_of(q):
+        _check(load_library().swm_rope_cache(
+            q_out.data_ptr(), q.data_ptr(), _opt_ptr(k), _opt_ptr(v), stride, positions.data_ptr(),
+            _opt_ptr(inv_freq) if rot else None, rot, None if k is None else key_cache.data_ptr(),
+            None if k is None else value_cache.data_ptr(), None if k is None else slot_mapping.data_ptr(), rows, heads,
+            kv_heads, dim, vdim, _act(q), _stream(q)))
+
+
+def group_router(h: torch.Tensor, router: torch.Tensor, correction: Optional[torch.Tensor], top: int, groups: int,
+                 keep: int, scale: float):
+    """-> (chosen int32 [rows, top], weights fp32 [rows, top])."""
+    _dev(h, router, correction)
+    _f32c(router, "router")
+    rows, width = h.shape
+    experts = router.shape[0]
+    _need(router.shape == (experts, width), "group_router: router shape")
+    if correction is not None:
+        _f32c(correction, "correction")
+        _need(correction.numel() == experts, "group_router: correction")
+    chosen = torch.empty(rows, top, dtype=torch.int32, device=h.device)
+    weights = torch.empty(rows, top, dtype=torch.float32, device=h.device)
+    with _on_device_of(h):
+        _check(load_library().swm_group_router(chosen.data_ptr(), weights.data_ptr(), h.data_ptr(), _rows(h, "h"),
+                                               router.data_ptr(), _opt_ptr(correction), rows, width, experts, top,
+                                               groups, keep, scale, _act(h), _stream(h)))
+    return chosen, weights
+
+
+def capped_attention(out: torch.Tensor, q: torch.Tensor, key_cache: torch.Tensor, value_cache: torch.Tensor,
+                     gate: Optional[torch.Tensor], batch, heads: int, kv_heads: int, dim: int, vdim: int, scale: float,
+                     softcap: float = 0.0, window: int = 0) -> None:
+    """out [rows, heads * vdim] (cache dtype); q fp32 [rows, heads * dim]; caches [pages, page, kv_heads * size];
+    gate (None: no gate): a 2-D view [rows, heads * vdim] in the cache dtype."""
+    _dev(out, q, key_cache, value_cache, gate)
+    _f32c(q, "q")
+    rows = q.shape[0]
+    n = _ragged_ok(batch, rows)
+    tables = batch.block_tables
+    _need(tables.dtype == torch.int32 and tables.is_contiguous() and tables.dim() == 2 and tables.shape[0] == n,
+          "capped_attention: block tables")
+    _need(q.shape[1] == heads * dim and out.shape == (rows, heads * vdim) and out.is_contiguous()
+          and out.dtype == key_cache.dtype == value_cache.dtype and key_cache.is_contiguous()
+          and value_cache.is_contiguous() and key_cache.shape[1:] == (value_cache.shape[1], kv_heads * dim)
+          and value_cache.shape[2] == kv_heads * vdim and key_cache.shape[0] == value_cache.shape[0],
+          "capped_attention: shapes")
+    _need(batch.max_pages_used <= tables.shape[1] and batch.max_page_id < key_cache.shape[0],
+          "capped_attention: block tables exceed the cache")
+    if gate is not None:
+        _need(gate.shape == out.shape and gate.dtype == out.dtype, "capped_attention: gate")
+    with _on_device_of(q):
+        _check(load_library().swm_capped_attention(
+            out.data_ptr(), q.data_ptr(), key_cache.data_ptr(), value_cache.data_ptr(), _opt_ptr(gate),
+            0 if gate is None else _rows(gate, "gate"), tables.data_ptr(), tables.shape[1], batch.q_start.data_ptr(),
+            batch.ctx_len.data_ptr(), rows, n, heads, kv_heads, dim, vdim, key_cache.shape[1], scale, softcap, window,
+            _act(out), _stream(q)))
+
+
+def lightning(out: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor,
+              state: torch.Tensor, batch, heads: int, dim: int, vdim: int) -> None:
+    """out fp32 [rows, heads * vdim]; q, k, v: column ranges of one projection output (before their silu);
+    decay fp32 [heads]; state fp32 [slots, heads, dim, vdim]."""
+    _dev(out, q, k, v, decay, state)
+    for t, what in ((out, "out"), (decay, "decay"), (state, "state")):
+        _f32c(t, what)
+    rows = q.shape[0]
+    n = _ragged_ok(batch, rows)
+    stride = _rows(q, "q")
+    _need(q.shape == (rows, heads * dim) and k.shape == q.shape and v.shape == (rows, heads * vdim)
+          and _rows(k, "k") == stride and _rows(v, "v") == stride and k.dtype == q.dtype and v.dtype == q.dtype
+          and out.shape == (rows, heads * vdim) and decay.numel() == heads and state.shape[1:] == (heads, dim, vdim)
+          and batch.max_state_slot < state.shape[0], "lightning: shapes")
+    with _on_device_of(q):
+        _check(load_library().swm_lightning(out.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), stride,
+                                            decay.data_ptr(), state.data_ptr(), batch.q_start.data_ptr(),
+                                            batch.ctx_len.data_ptr(), batch.state_slot.data_ptr(), rows, n, heads, dim,
+                                            vdim, _act(q), _stream(q)))
+
+
+ops = SimpleNamespace(expert_ffn=expert_ffn, ACT_GELU=ACT_GELU, ACT_RELU2=ACT_RELU2,
     scalar_norm_add=scalar_norm_add, scalar_norm=scalar_norm, qk_norm_cache=qk_norm_cache,
     window_attention=window_attention, short_conv=short_conv, channel_delta=channel_delta,
-    general_delta=general_delta, head_norm_gate=head_norm_gate)
+    general_delta=general_delta, head_norm_gate=head_norm_gate, stream_add_norm=stream_add_norm,
+    clamped_glu=clamped_glu, relu2=relu2, rope_cache=rope_cache, group_router=group_router,
+    capped_attention=capped_attention, lightning=lightning)

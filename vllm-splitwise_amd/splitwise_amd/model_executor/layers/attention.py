@@ -260,3 +260,44 @@ class WindowTalkingAttention(nn.Module):
         _C.mixer_ops.window_attention(out, q32, key_cache, value_cache, self.talk.data, md.ragged, self.heads,
                                       self.kv_heads, self.dim, self.vdim, self.scale, self.window, self.keep_first)
         return out
+
+
+class CappedGatedAttention(nn.Module):
+    """Causal softmax attention with grouped query heads over a paged cache, for models that want scores,
+    weights and positions in fp32:  partial rotary embedding on neighbouring pairs (frequencies given as a table,
+    angles from fp32 positions) on q and k, score = (q . k) * scale, optionally softcap * tanh(score / softcap),
+    optionally a sliding window, and optionally a sigmoid gate on the concatenated heads (the gate is a projection
+    of the same input as q).  Keys are cached AFTER rotation; a layer built with ``shares_kv`` has no key / value
+    projections and reads the cache of the layer it names with its own queries.  Caches are
+    [pages, page, kv_heads * size], token-major inside a page."""
+
+    def __init__(self, heads: int, kv_heads: int, dim: int, vdim: int, scale: float, softcap: float = 0.0,
+                 inv_freq: Optional[torch.Tensor] = None, window: int = 0, shares_kv: bool = False) -> None:
+        super().__init__()
+        assert heads % kv_heads == 0
+        self.heads, self.kv_heads, self.dim, self.vdim = heads, kv_heads, dim, vdim
+        self.scale, self.softcap, self.window, self.shares_kv = float(scale), float(softcap or 0.0), int(window), shares_kv
+        freqs = torch.zeros(0, dtype=torch.float32) if inv_freq is None else inv_freq.to(torch.float32)
+        assert 2 * freqs.numel() <= dim
+        self.register_buffer("inv_freq", freqs.clone(), persistent=False)     # a constant of the config, not a weight
+
+    def cache_shapes(self, block_size: int):
+        """Per page: keys, values."""
+        return [(block_size, self.kv_heads * self.dim), (block_size, self.kv_heads * self.vdim)]
+
+    def forward(self, q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.Tensor],
+                gate: Optional[torch.Tensor], positions: torch.Tensor, key_cache: torch.Tensor,
+                value_cache: torch.Tensor, md: InputMetadata) -> torch.Tensor:
+        """q, k, v, gate: column ranges of one projection output [rows, *]; k, v None for a layer that shares them."""
+        rows = q.shape[0]
+        q32 = torch.empty(rows, self.heads * self.dim, dtype=torch.float32, device=q.device)
+        if self.shares_kv:
+            _C.mixer_ops.rope_cache(q32, q, None, None, positions, self.inv_freq, self.heads, self.kv_heads,
+                                    self.dim, self.vdim, None, None, None)
+        else:
+            _C.mixer_ops.rope_cache(q32, q, k, v, positions, self.inv_freq, self.heads, self.kv_heads, self.dim,
+                                    self.vdim, key_cache, value_cache, md.slot_mapping)
+        out = torch.empty(rows, self.heads * self.vdim, dtype=q.dtype, device=q.device)
+        _C.mixer_ops.capped_attention(out, q32, key_cache, value_cache, gate, md.ragged, self.heads, self.kv_heads,
+                                      self.dim, self.vdim, self.scale, self.softcap, self.window)
+        return out

@@ -5,6 +5,7 @@ Each layer keeps the reference's two entry points: ``forward`` (native kernel) a
 vllm/model_executor/layers/layernorm.py:10-65, rotary_embedding.py:36-141,
 activation.py:15-44.
 """
+import math
 from typing import Optional, Tuple, Union
 
 import torch
@@ -124,4 +125,82 @@ class ScalarRMSNorm(nn.Module):
         """The model's final norm: fp32 stream in, activations out."""
         out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
         _C.mixer_ops.scalar_norm(out, x, self.weight.data, self.variance_epsilon)
+        return out
+
+
+class OffsetRMSNorm(nn.Module):
+    """RMS norm of an fp32 residual stream with a per-channel weight stored as a difference from ``offset``:
+    out = x / sqrt(mean(x^2) + eps) * (offset + w).  ``add_norm`` first sums sublayer outputs into the stream
+    (x += a + b + c, the addends summed first), so a layer whose sublayers run side by side on one norm costs one
+    pass over the stream per layer.  The weight is kept in fp32."""
+
+    def __init__(self, width: int, eps: float = 1e-6, offset: float = 1.0) -> None:
+        super().__init__()
+        self.weight = nn.Parameter(torch.zeros(width, dtype=torch.float32), requires_grad=False)
+        self.variance_epsilon, self.offset = eps, float(offset)
+
+    def _forward(self, x: torch.Tensor) -> torch.Tensor:
+        x = x.float()
+        return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + self.variance_epsilon) * (self.offset + self.weight)
+
+    def add_norm(self, residual: torch.Tensor, out_dtype: torch.dtype, a: Optional[torch.Tensor] = None,
+                 b: Optional[torch.Tensor] = None, c: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """``residual`` fp32, updated in place; a, b: sublayer outputs in ``out_dtype``; c: an fp32 one."""
+        out = torch.empty(residual.shape, dtype=out_dtype, device=residual.device)
+        _C.mixer_ops.stream_add_norm(residual, self.weight.data, self.offset, self.variance_epsilon, out, a, b, c)
+        return out
+
+    def forward(self, x: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+        return self.add_norm(x, out_dtype)
+
+
+def scaled_rotary_frequencies(rot_dims: int, base: float, scaling: Optional[dict] = None) -> torch.Tensor:
+    """fp32 [rot_dims / 2]: f_i = base^(-2i / rot_dims), with long waves slowed down as Llama 3.1 does it
+    (``scaling``: factor, low, high, original): a wavelength below original / high keeps f, one above original / low
+    gets f / factor, between the two the mix (1 - s) f / factor + s f with s = (original / wavelength - low) /
+    (high - low).  Worked out in double precision, rounded once."""
+    out = []
+    for i in range(rot_dims // 2):
+        f = float(base) ** (-2.0 * i / rot_dims)
+        if scaling:
+            wavelength = 2.0 * math.pi / f
+            original, low, high = scaling["original"], scaling["low"], scaling["high"]
+            if wavelength < original / high:
+                pass
+            elif wavelength > original / low:
+                f /= scaling["factor"]
+            else:
+                s = (original / wavelength - low) / (high - low)
+                f = (1.0 - s) * f / scaling["factor"] + s * f
+        out.append(f)
+    return torch.tensor(out, dtype=torch.float64).to(torch.float32)
+
+
+class ClampedGLU(nn.Module):
+    """Gated activation with limits: x = gate | up;  g = min(gate, limit), u = clamp(up, -limit, limit);
+    out = g * sigmoid(alpha * g) * (u + shift).  alpha = 1.702 makes g sigmoid(alpha g) the sigmoid form of gelu."""
+
+    def __init__(self, alpha: float = 1.702, limit: float = math.inf, shift: float = 1.0) -> None:
+        super().__init__()
+        self.alpha, self.limit, self.shift = float(alpha), float(limit), float(shift)
+
+    def _forward(self, x: torch.Tensor) -> torch.Tensor:
+        d = x.shape[-1] // 2
+        g = x[..., :d].float().clamp(max=self.limit)
+        u = x[..., d:].float().clamp(-self.limit, self.limit)
+        return (g * torch.sigmoid(self.alpha * g) * (u + self.shift)).to(x.dtype)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        out = torch.empty(x.shape[0], x.shape[1] // 2, dtype=x.dtype, device=x.device)
+        _C.mixer_ops.clamped_glu(out, x, self.alpha, self.limit, self.shift)
+        return out
+
+
+class ReluSquared(nn.Module):
+    def _forward(self, x: torch.Tensor) -> torch.Tensor:
+        return torch.relu(x).pow(2)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+        _C.mixer_ops.relu2(out, x)
         return out

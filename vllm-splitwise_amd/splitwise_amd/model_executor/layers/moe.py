@@ -4,17 +4,22 @@
 expert weighs 1 / top.  An expert is down(gelu(up x)) with the exact (erf) gelu and no biases.  An optional
 shared expert of the same form runs for every token and is added after a per-token sigmoid gate.
 
+``GroupRoutedExperts``: a learned sigmoid router in fp32 with a selection bias that enters the choice but not the
+weights, a choice limited to the best groups of neighbouring experts, weights normalised over the chosen experts
+and scaled; an expert is down(relu(up x)^2); an optional shared expert of the same form is returned beside the
+routed sum so that the caller's residual add can take both.
+
 Rows are grouped by expert on the device (a stable sort of the (row, choice) pairs by expert id, then a binary
 search for every expert's first pair), so each expert's rows are one contiguous run and the host never waits.
 """
-from typing import Dict, Optional
+from typing import Dict, Optional, Tuple
 
 import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
 from ... import _C
-from .linear import MergedColumnParallelLinear, RowParallelLinear
+from .linear import ColumnParallelLinear, MergedColumnParallelLinear, RowParallelLinear
 
 
 class TableRoutedExperts(nn.Module):
@@ -60,4 +65,58 @@ class TableRoutedExperts(nn.Module):
         self.down.data.copy_(torch.stack([w[f"e{e}.down"] for e in range(self.num_experts)]))
         if self.shared_ff:
             self.shared_in.weight.data.copy_(torch.cat([w["shared.up"], w["shared.sg"]], 0))
+            self.shared_down.weight.data.copy_(w["shared.down"])
+
+
+def group_pairs_by_expert(experts: torch.Tensor, num_experts: int):
+    """experts int32 [rows, top] -> (order int32 [rows * top]: pair index row * top + choice sorted by expert,
+    expert_start int32 [experts + 1]); all on the device."""
+    flat = experts.reshape(-1)
+    by_expert, order = torch.sort(flat, stable=True)
+    edges = torch.arange(num_experts + 1, dtype=flat.dtype, device=flat.device)
+    return order.to(torch.int32), torch.searchsorted(by_expert, edges).to(torch.int32)
+
+
+class GroupRoutedExperts(nn.Module):
+    def __init__(self, width: int, num_experts: int, top: int, ff: int, shared_ff: Optional[int], groups: int,
+                 keep_groups: int, scale: float, dtype: torch.dtype, linear_method=None) -> None:
+        super().__init__()
+        if num_experts % groups != 0 or not (1 <= keep_groups <= groups) or keep_groups * (num_experts // groups) < top:
+            raise ValueError(f"{num_experts} experts in {groups} groups with {keep_groups} kept cannot give {top} choices")
+        self.width, self.num_experts, self.top, self.ff = width, num_experts, top, ff
+        self.groups, self.keep_groups, self.scale = groups, keep_groups, float(scale)
+        # the router is fp32 whatever the model's dtype
+        self.router = nn.Parameter(torch.zeros(num_experts, width, dtype=torch.float32), requires_grad=False)
+        self.correction = nn.Parameter(torch.zeros(num_experts, dtype=torch.float32), requires_grad=False)
+        self.up = nn.Parameter(torch.empty(num_experts, ff, width, dtype=dtype), requires_grad=False)
+        self.down = nn.Parameter(torch.empty(num_experts, width, ff, dtype=dtype), requires_grad=False)
+        self.shared_ff = shared_ff
+        if shared_ff:
+            self.shared_up = ColumnParallelLinear(width, shared_ff, False, dtype, linear_method)
+            self.shared_down = RowParallelLinear(shared_ff, width, False, dtype, linear_method)
+
+    def forward(self, h: torch.Tensor) -> Tuple[Optional[torch.Tensor], torch.Tensor]:
+        """-> (shared expert's output in h's dtype or None, routed experts' weighted sum in fp32)."""
+        chosen, weights = _C.mixer_ops.group_router(h, self.router.data, self.correction.data, self.top, self.groups,
+                                                    self.keep_groups, self.scale)
+        order, start = group_pairs_by_expert(chosen, self.num_experts)
+        out = torch.zeros(h.shape[0], self.width, dtype=torch.float32, device=h.device)
+        _C.mixer_ops.expert_ffn(out, h, self.up.data, self.down.data, order, start, self.top, 1.0,
+                                activation=_C.mixer_ops.ACT_RELU2, pair_weight=weights)
+        shared = None
+        if self.shared_ff:
+            hidden = self.shared_up(h)
+            act = torch.empty_like(hidden)
+            _C.mixer_ops.relu2(act, hidden)
+            shared = self.shared_down(act)
+        return shared, out
+
+    def load_named(self, w: Dict[str, torch.Tensor]) -> None:
+        self.router.data.copy_(w["router"].float())
+        if "correction" in w:
+            self.correction.data.copy_(w["correction"].float())
+        self.up.data.copy_(torch.stack([w[f"e{e}.up"] for e in range(self.num_experts)]))
+        self.down.data.copy_(torch.stack([w[f"e{e}.down"] for e in range(self.num_experts)]))
+        if self.shared_ff:
+            self.shared_up.weight.data.copy_(w["shared.up"])
             self.shared_down.weight.data.copy_(w["shared.down"])

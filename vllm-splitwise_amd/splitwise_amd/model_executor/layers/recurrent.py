@@ -11,8 +11,12 @@ Delta rule, per head, S [key size, value size] (keys index rows):
                           g = exp(-exp(A_log) softplus(low-rank(h) + dt_bias)) per head and key channel
   ``GeneralDeltaMixer``   S <- diag(w) S - (a * u)(u^T S) + k v^T;  o = S^T r,  u = k / |k|
                           w = exp(-e^(-1/2) sigmoid(low-rank-tanh(h) + w0)),  a = sigmoid(W_a h + b)
+
+Linear attention, per head, S [key size, value size]:
+  ``LightningMixer``      S <- decay_h S + k v^T;  o = S^T q,  q, k, v = silu of their projections; the heads'
+                          outputs are normed together, gated by a sigmoid and projected
 """
-from typing import Dict, List, Tuple
+from typing import Dict, List, Sequence, Tuple
 
 import torch
 import torch.nn as nn
@@ -118,4 +122,43 @@ class GeneralDeltaMixer(nn.Module):
         self.o_proj.weight.data.copy_(w["o"])
         self.w0.data.copy_(w["w0"].float())
         self.rate_bias.data.copy_(w["a.b"].float())
+        self.out_norm.data.copy_(w["norm"].float())
+
+
+class LightningMixer(nn.Module):
+    """Linear attention with one constant decay per head.  q | k | v | gate are one GEMM of the layer's input; the
+    recurrence runs in fp32 on the silu of q, k, v (chunks of 32 tokens as matrix products); the concatenated heads
+    get ONE RMS norm over all of them (weight [heads * vdim]), times sigmoid(gate), then the output projection."""
+
+    def __init__(self, width: int, heads: int, dim: int, vdim: int, decay: Sequence[float], eps: float,
+                 dtype: torch.dtype, linear_method=None) -> None:
+        super().__init__()
+        assert len(decay) == heads
+        self.heads, self.dim, self.vdim, self.eps = heads, dim, vdim, eps
+        self.in_sizes = [heads * dim, heads * dim, heads * vdim, heads * vdim]
+        self.in_proj = MergedColumnParallelLinear(width, self.in_sizes, False, dtype, linear_method)
+        self.o_proj = RowParallelLinear(heads * vdim, width, False, dtype, linear_method)
+        # a constant of the config, not a weight
+        self.register_buffer("decay", torch.tensor([float(d) for d in decay], dtype=torch.float64).to(torch.float32),
+                             persistent=False)
+        self.out_norm = nn.Parameter(torch.ones(heads * vdim, dtype=torch.float32), requires_grad=False)
+
+    def state_shapes(self) -> List[Tuple[int, ...]]:
+        return [(self.heads, self.dim, self.vdim)]
+
+    def forward(self, h: torch.Tensor, state: List[torch.Tensor], md: InputMetadata) -> torch.Tensor:
+        rows = h.shape[0]
+        proj = self.in_proj(h)
+        nk, nv = self.heads * self.dim, self.heads * self.vdim
+        o = torch.empty(rows, nv, dtype=torch.float32, device=h.device)
+        _C.mixer_ops.lightning(o, proj[:, :nk], proj[:, nk:2 * nk], proj[:, 2 * nk:2 * nk + nv], self.decay,
+                               state[0], md.ragged, self.heads, self.dim, self.vdim)
+        gated = torch.empty(rows, nv, dtype=h.dtype, device=h.device)
+        # one "head" of heads * vdim channels: the norm runs over all heads together
+        _C.mixer_ops.head_norm_gate(gated, o, proj[:, 2 * nk + nv:], self.out_norm.data, True, self.eps, 1, nv)
+        return self.o_proj(gated)
+
+    def load_named(self, w: Dict[str, torch.Tensor]) -> None:
+        self.in_proj.weight.data.copy_(torch.cat([w["q"], w["k"], w["v"], w["g"]], 0))
+        self.o_proj.weight.data.copy_(w["o"])
         self.out_norm.data.copy_(w["norm"].float())

@@ -13,11 +13,13 @@ import torch
 import torch.nn as nn
 
 from ..config import ModelConfig
+from .models.lapilorn import LapilornForCausalLM
 from .models.llama import LlamaForCausalLM
 from .models.nepevik import NepevikForCausalLM
 from .models.opt import OPTForCausalLM
 
-_ARCH = {"llama": LlamaForCausalLM, "opt": OPTForCausalLM, "nepevik": NepevikForCausalLM}
+_ARCH = {"llama": LlamaForCausalLM, "opt": OPTForCausalLM, "nepevik": NepevikForCausalLM,
+         "lapilorn": LapilornForCausalLM}
 
 
 def architecture_class(name: str):
