@@ -112,10 +112,12 @@ def parse_args():
                     help="N > 1: legs after the headline leg are skipped once the run has taken this long")
     ap.add_argument("--leg-timeout", type=float, default=600.0, help="N > 1: longest any one leg may take (s)")
     ap.add_argument("--mixers", action="store_true",
-                    help="instead of the headline workload: prefill / decode throughput of a Nepevik stack beside a Llama "
+                    help="instead of the headline workload: prefill / decode throughput of a Nepevik (or, with --mixer-family, Lapilorn) stack beside a Llama "
                          "stack of equal size (random weights), and the mixer kernels beside the like Llama kernels with "
                          "their distances from the roofline; one JSON line")
     ap.add_argument("--mixer-sizes", default="2k", help="with --mixers: comma-separated preset sizes (2k, 4k)")
+    ap.add_argument("--mixer-family", default="nepevik", choices=["nepevik", "lapilorn"],
+                    help="with --mixers: the family of listed-layer decoders to measure beside Llama")
     ap.add_argument("--replica", default=None, help=argparse.SUPPRESS)          # set by the launcher
     ap.add_argument("--worker-cls", default=None, help=argparse.SUPPRESS)       # CPU dry runs of the launcher
     return ap.parse_args()
@@ -376,8 +378,8 @@ def cpu_baseline(model_name, prompt_len, decode_len):
 
 def mixers_bench(args) -> None:
     from splitwise_amd.executor import bench_mixers
-    result = bench_mixers.run(tuple(x for x in args.mixer_sizes.split(",") if x))
-    print(json.dumps({"metric": "nepevik_vs_llama_throughput", "unit": "tok/s", "n_gpus": 1, "dtype": "bf16",
+    result = bench_mixers.run(tuple(x for x in args.mixer_sizes.split(",") if x), family=args.mixer_family)
+    print(json.dumps({"metric": f"{args.mixer_family}_vs_llama_throughput", "unit": "tok/s", "n_gpus": 1, "dtype": "bf16",
                       "data": "synthetic", **result}))
 
 

@@ -65,6 +65,37 @@ _NEPEVIK_PRESETS = {
     "nepevik-2k": (2048, 2, 16, 4, 32, 2, 1024),
     "nepevik-4k": (4096, 2, 32, 8, 32, 2, 2048),
 }
+
+
+def _lapilorn_preset(width: int, repeats: int, heads: int, kv_heads: int, experts: int, top: int, ff: int) -> dict:
+    """A Lapilorn stack of layer sizes that resemble a served model's: per repeat an attention layer with keys of its
+    own and a dense feed-forward, a lightning layer with routed experts, an attention layer that reads the first
+    one's keys, another lightning layer, and a lightning layer without a feed-forward."""
+    d = width // heads
+    rot = {"base": 500000.0, "dims": d // 2, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}
+    attn = {"heads": heads, "kv_heads": kv_heads, "dim": d, "vdim": d, "scale": d ** -0.5, "softcap": 30.0, "rot": rot}
+    light = {"heads": heads, "dim": d, "vdim": d, "decay": [1.0 - 2.0 ** (-3 - 5 * i / max(heads - 1, 1)) for i in range(heads)]}
+    dense = {"kind": "dense", "ff": (11 * ff) // 4, "limit": 7.0}
+    moe = {"kind": "moe", "expert": {"ff": ff}, "shared": {"ff": ff},
+           "router": {"experts": experts, "top": top, "scale": 2.5, "groups": {"count": 4, "keep": 2}}}
+    layers = []
+    for _ in range(repeats):
+        first = len(layers)
+        layers += [{"type": "attention", "mixer": dict(attn), "mlp": dense},
+                   {"type": "lightning", "mixer": dict(light), "mlp": moe},
+                   {"type": "attention", "mixer": dict(attn, kv_from=first), "mlp": dense},
+                   {"type": "lightning", "mixer": dict(light), "mlp": moe},
+                   {"type": "lightning", "mixer": dict(light), "mlp": None}]
+    from .model_executor.models.lapilorn import normalize_config
+    return normalize_config({"architecture": "Lapilorn", "layers": layers, "norm": {"eps": 1e-6}, "vocab": 32000,
+                             "width": width})
+
+
+_LAPILORN_PRESETS = {
+    # name: (width, repeats of the 5-layer pattern, heads, kv heads, experts, top, expert ff)
+    "lapilorn-2k": (2048, 2, 16, 4, 32, 2, 1024),
+    "lapilorn-4k": (4096, 2, 32, 8, 32, 2, 2048),
+}
 # Llama stacks of the same width, depth and active feed-forward size, to measure the above against
 MODEL_PRESETS.update({
     "llama-2k": dict(architecture="llama", vocab_size=32000, hidden_size=2048, num_hidden_layers=10,
@@ -123,6 +154,8 @@ class ModelConfig:
             return dict(MODEL_PRESETS[name])
         if name in _NEPEVIK_PRESETS:
             return _nepevik_preset(*_NEPEVIK_PRESETS[name])
+        if name in _LAPILORN_PRESETS:
+            return _lapilorn_preset(*_LAPILORN_PRESETS[name])
         cfg_path = os.path.join(model, "config.json")
         if os.path.isfile(cfg_path):
             with open(cfg_path) as f:

@@ -1,4 +1,4 @@
-"""Throughput of a Nepevik stack beside a Llama stack of the same width, depth and active feed-forward size
+"""Throughput of a Nepevik (or Lapilorn) stack beside a Llama stack of the same width, depth and active feed-forward size
 (random weights), and every mixer kernel beside the like kernel of the Llama path with their distances from
 the roofline.  ``bench.py --mixers`` prints the result as one JSON line.
 
@@ -246,13 +246,165 @@ def kernel_table(width: int = 2048, heads: int = 16, kv_heads: int = 4, window: 
     return rows
 
 
-def run(sizes=("2k",), with_kernels: bool = True) -> dict:
-    result = {"engine": {}, "kernels": {}}
+@torch.inference_mode()
+def kernel_table_lapilorn(width: int = 2048, heads: int = 16, kv_heads: int = 4, prefill_rows: int = 4096,
+                          decode_seqs: int = 64, decode_ctx: int = 2048, experts: int = 32, top: int = 2,
+                          ff: int = 1024) -> List[dict]:
+    """The kernels of the Lapilorn layers beside the like kernels of the Llama path (or, for the recurrence, of the
+    delta-rule layers).  fp32 matrix work (scores, softmax weights and states must stay fp32) is priced at the fp32
+    matrix peak, which equals the fp32 vector peak on this GPU."""
+    from .. import _C
+    dev, bf = torch.device("cuda"), torch.bfloat16
+    d = width // heads
+    page = 16
+    rows: List[dict] = []
+    scale = d ** -0.5
+    for phase, seqs in (("prefill", [(0, prefill_rows // 2, 0, None), (0, prefill_rows // 2, 1, None)]),
+                        ("decode", [(decode_ctx, 1, i, None) for i in range(decode_seqs)])):
+        total_pages, laid = 0, []
+        for ctx, n, slot, _ in seqs:
+            pages = -(-(ctx + n) // page)
+            laid.append((ctx, n, slot, list(range(total_pages, total_pages + pages))))
+            total_pages += pages
+        batch = _ragged(laid, dev)
+        T, B = sum(s[1] for s in laid), len(laid)
+        # ---------------------------------------------------------------- attention
+        kc = torch.randn(total_pages, page, kv_heads * d, device=dev).to(bf)
+        vc = torch.randn(total_pages, page, kv_heads * d, device=dev).to(bf)
+        q = torch.randn(T, heads * d, device=dev)
+        gate = torch.randn(T, heads * d, device=dev).to(bf)
+        out = torch.empty(T, heads * d, dtype=bf, device=dev)
+        t = _time(lambda: _C.mixer_ops.capped_attention(out, q, kc, vc, gate, batch, heads, kv_heads, d, d, scale, 30.0, 0))
+        pairs = sum(c + i + 1 for c, n, _, _ in laid for i in range(n))
+        keys = sum(c + n for c, n, _, _ in laid)
+        rows.append(_row("capped_attention (fp32 matrix cores, gate fused)", phase, t,
+                         keys * kv_heads * d * 2 * 2 + T * heads * d * (4 + 2 + 2), 4.0 * pairs * heads * d, VALU_F32))
+        if phase == "prefill":
+            qh = torch.randn(T, heads, d, device=dev).to(bf)
+            kh = torch.randn(T, kv_heads, d, device=dev).to(bf)
+            vh = torch.randn(T, kv_heads, d, device=dev).to(bf)
+            oh = torch.empty_like(qh)
+            starts = torch.tensor([0, T // 2], dtype=torch.int32, device=dev)
+            lens = torch.tensor([T // 2, T // 2], dtype=torch.int32, device=dev)
+            t2 = _time(lambda: _C.ops.prefill_attention(oh, qh, kh, vh, starts, lens, T // 2, scale, None, None))
+            rows.append(_row("Llama prefill_attention (bf16 matrix cores)", phase, t2,
+                             T * (heads + 2 * kv_heads) * d * 2 + T * heads * d * 2, 4.0 * pairs * heads * d, MFMA_BF16,
+                             like="capped_attention"))
+        else:
+            x = 8
+            per_seq = -(-(decode_ctx + 1) // page)
+            nb = decode_seqs * per_seq + 1
+            kc2 = torch.randn(nb, kv_heads, d // x, page, x, device=dev).to(bf)
+            vc2 = torch.randn(nb, kv_heads, d, page, device=dev).to(bf)
+            bt = torch.randperm(nb - 1, device=dev).to(torch.int32).view(decode_seqs, -1).contiguous()
+            cl = torch.full((decode_seqs,), decode_ctx + 1, dtype=torch.int32, device=dev)
+            qh = torch.randn(decode_seqs, heads, d, device=dev).to(bf)
+            oh = torch.empty_like(qh)
+            t2 = _time(lambda: _C.ops.paged_attention_v1(oh, qh, kc2, vc2, kv_heads, scale, bt, cl, page, decode_ctx + 1,
+                                                         None, "auto"))
+            rows.append(_row("Llama paged_attention_v1", phase, t2,
+                             decode_seqs * (decode_ctx + 1) * kv_heads * d * 2 * 2 + 2 * decode_seqs * heads * d * 2,
+                             4.0 * decode_seqs * (decode_ctx + 1) * heads * d, VALU_F32, like="capped_attention"))
+        # ---------------------------------------------------------------- rotation + cache write
+        proj = torch.randn(T, (heads + 2 * kv_heads) * d, device=dev).to(bf)
+        pos = torch.cat([torch.arange(c, c + n) for c, n, _, _ in laid]).to(dev)
+        slots = torch.cat([torch.tensor([tb[p // page] * page + p % page for p in range(c, c + n)])
+                           for c, n, _, tb in laid]).to(dev)
+        inv = torch.rand(d // 4, device=dev)
+        q32 = torch.empty(T, heads * d, device=dev)
+        t = _time(lambda: _C.mixer_ops.rope_cache(q32, proj[:, :heads * d], proj[:, heads * d:(heads + kv_heads) * d],
+                                                  proj[:, (heads + kv_heads) * d:], pos, inv, heads, kv_heads, d, d, kc, vc,
+                                                  slots))
+        rows.append(_row("rope_cache (fp32 angles, fp32 queries out)", phase, t,
+                         T * ((heads + 2 * kv_heads) * d * 2 + heads * d * 4 + 2 * kv_heads * d * 2), 6.0 * T * heads * d,
+                         VALU_F32))
+        # ---------------------------------------------------------------- lightning / delta rule
+        lseqs = [(c, n, i, []) for i, (c, n, _, _) in enumerate(laid)]
+        lbatch = _ragged(lseqs, dev)
+        lproj = torch.randn(T, 3 * heads * d, device=dev).to(bf)
+        state = torch.zeros(max(B, 2), heads, d, d, device=dev)
+        decay = torch.full((heads,), 0.97, device=dev)
+        lo = torch.empty(T, heads * d, device=dev)
+        t = _time(lambda: _C.mixer_ops.lightning(lo, lproj[:, :heads * d], lproj[:, heads * d:2 * heads * d],
+                                                 lproj[:, 2 * heads * d:], decay, state, lbatch, heads, d, d))
+        chunk = 32
+        lflops = T * heads * (2.0 * chunk * d + 2.0 * chunk * d + 4.0 * d * d)      # in-chunk scores and sums, state in and out
+        lbytes = T * heads * d * (3 * 2 + 4) + 2 * B * heads * d * d * 4
+        rows.append(_row("lightning (chunks of 32 on fp32 matrix cores)", phase, t, lbytes, lflops, VALU_F32))
+        qkv = torch.randn(T, 3 * heads * d, device=dev)
+        beta = torch.randn(T, heads, device=dev).to(bf)
+        dpre = torch.randn(T, heads * d, device=dev).to(bf)
+        o = torch.empty(T, heads * d, device=dev)
+        dt_bias, a_log = torch.zeros(heads * d, device=dev), torch.zeros(heads, device=dev)
+        t2 = _time(lambda: _C.mixer_ops.channel_delta(o, qkv, beta, dpre, dt_bias, a_log, state, lbatch, heads, heads, d, d))
+        rows.append(_row("Nepevik channel_delta (token by token)", phase, t2,
+                         T * (3 * heads * d * 4 + heads * d * 2 + heads * d * 4) + 2 * B * heads * d * d * 4,
+                         8.0 * T * heads * d * d, VALU_F32, like="lightning"))
+        # ---------------------------------------------------------------- whole-heads norm and gate
+        gated = torch.empty(T, heads * d, dtype=bf, device=dev)
+        wn = torch.ones(heads * d, device=dev)
+        t = _time(lambda: _C.mixer_ops.head_norm_gate(gated, lo, gate, wn, True, 1e-6, 1, heads * d))
+        rows.append(_row("head_norm_gate (one norm over all heads)", phase, t, T * heads * d * (4 + 2 + 2), 6.0 * T * heads * d,
+                         VALU_F32))
+        # ---------------------------------------------------------------- residual add + next norm
+        res = torch.randn(T, width, device=dev)
+        a = torch.randn(T, width, device=dev).to(bf)
+        b2 = torch.randn(T, width, device=dev).to(bf)
+        c32 = torch.randn(T, width, device=dev)
+        hout = torch.empty(T, width, dtype=bf, device=dev)
+        wgt = torch.zeros(width, device=dev)
+        t = _time(lambda: _C.mixer_ops.stream_add_norm(res, wgt, 1.0, 1e-6, hout, a, b2, None))
+        rows.append(_row("stream_add_norm (fp32 stream, two addends)", phase, t, T * width * (4 + 4 + 2 + 2 + 2), 6.0 * T * width,
+                         VALU_F32))
+        t = _time(lambda: _C.mixer_ops.stream_add_norm(res, wgt, 1.0, 1e-6, hout, a, b2, c32))
+        rows.append(_row("stream_add_norm (three addends, one fp32)", phase, t, T * width * (4 + 4 + 2 + 2 + 4 + 2), 7.0 * T * width,
+                         VALU_F32))
+        xr, rr, wr = a.clone(), a.clone(), torch.ones(width, dtype=bf, device=dev)
+        t2 = _time(lambda: _C.ops.fused_add_rms_norm(xr, rr, wr, 1e-6))
+        rows.append(_row("Llama fused_add_rms_norm (bf16 stream)", phase, t2, T * width * 2 * 4, 4.0 * T * width, VALU_F32,
+                         like="stream_add_norm"))
+        # ---------------------------------------------------------------- gated activation
+        dff = (11 * ff) // 4
+        gu = torch.randn(T, 2 * dff, device=dev).to(bf)
+        act = torch.empty(T, dff, dtype=bf, device=dev)
+        t = _time(lambda: _C.mixer_ops.clamped_glu(act, gu, 1.702, 7.0, 1.0))
+        rows.append(_row("clamped_glu", phase, t, T * dff * 3 * 2, 8.0 * T * dff, VALU_F32))
+        t2 = _time(lambda: _C.ops.silu_and_mul(act, gu))
+        rows.append(_row("Llama silu_and_mul", phase, t2, T * dff * 3 * 2, 5.0 * T * dff, VALU_F32, like="clamped_glu"))
+        # ---------------------------------------------------------------- router and experts
+        hin = torch.randn(T, width, device=dev).to(bf)
+        router = torch.randn(experts, width, device=dev) * width ** -0.5
+        corr = torch.randn(experts, device=dev) * 0.1
+        t = _time(lambda: _C.mixer_ops.group_router(hin, router, corr, top, 4, 2, 2.5))
+        rows.append(_row("group_router (fp32)", phase, t, T * width * 2 + experts * width * 4 + T * top * 8,
+                         2.0 * T * experts * width, VALU_F32))
+        chosen, weights = _C.mixer_ops.group_router(hin, router, corr, top, 4, 2, 2.5)
+        from ..model_executor.layers.moe import group_pairs_by_expert
+        order, start = group_pairs_by_expert(chosen, experts)
+        up = torch.randn(experts, ff, width, device=dev).to(bf) * 0.02
+        down = torch.randn(experts, width, ff, device=dev).to(bf) * 0.02
+        eo = torch.zeros(T, width, device=dev)
+        t = _time(lambda: _C.mixer_ops.expert_ffn(eo, hin, up, down, order, start, top, 1.0,
+                                                  activation=_C.mixer_ops.ACT_RELU2, pair_weight=weights))
+        flops = 4.0 * T * top * ff * width
+        touched = min(experts, T * top)
+        rows.append(_row("expert_ffn (grouped, relu^2, weighted)", phase, t,
+                         touched * 2 * ff * width * 2 + T * width * (2 + 4) + T * top * ff * 2 * 2, flops, MFMA_BF16))
+        w1 = torch.randn(top * ff, width, device=dev).to(bf) * 0.02
+        w2 = torch.randn(width, top * ff, device=dev).to(bf) * 0.02
+        t2 = _time(lambda: torch.nn.functional.linear(torch.nn.functional.gelu(torch.nn.functional.linear(hin, w1)), w2))
+        rows.append(_row("dense feed-forward of the same active size (library GEMMs)", phase, t2,
+                         2 * top * ff * width * 2 + T * width * 4 + T * top * ff * 4, flops, MFMA_BF16, like="expert_ffn"))
+    return rows
+
+
+def run(sizes=("2k",), with_kernels: bool = True, family: str = "nepevik") -> dict:
+    result = {"family": family, "engine": {}, "kernels": {}}
     for size in sizes:
         pair = {}
-        for family in ("nepevik", "llama"):
-            pair[family] = {k: round(v, 2) for k, v in engine_throughput(f"{family}-{size}").items()}
+        for name in (family, "llama"):
+            pair[name] = {k: round(v, 2) for k, v in engine_throughput(f"{name}-{size}").items()}
         result["engine"][size] = pair
     if with_kernels:
-        result["kernels"]["2k"] = kernel_table()
+        result["kernels"]["2k"] = kernel_table() if family == "nepevik" else kernel_table_lapilorn()
     return result
