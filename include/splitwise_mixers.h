@@ -167,26 +167,26 @@ int swm_rope_cache(float* q_out, const void* q, const void* k, const void* v, in
                    const int64_t* slot_mapping, int64_t rows, int heads, int kv_heads, int dim, int vdim, int act_dtype,
                    void* stream);
 
-/* Router of a mixture of experts: s = sigmoid(router h) in fp32 (router fp32 [experts, width]); choice scores
- * s + correction (NULL: none); experts form `groups` equal groups of neighbours, a group scores the sum of its two
- * largest choice scores and only the best `keep` groups stay in the choice (groups == 1 or keep == groups: all);
- * the `top` largest choice scores are chosen; weights = s of the chosen / (their sum + 1e-20) * scale.
- * chosen int32 [rows, top], weights fp32 [rows, top]. */
-int swm_group_router(int32_t* chosen, float* weights, const void* h, int64_t h_stride, const float* router,
-                     const float* correction, int64_t rows, int width, int experts, int top, int groups, int keep,
-                     float scale, int act_dtype, void* stream);
+/* The choice of a mixture-of-experts router from its logits (fp32 [rows, experts], the router's product with the
+ * layer input): s = sigmoid(logit); choice scores s + correction (NULL: none); experts form `groups` equal groups
+ * of neighbours, a group scores the sum of its two largest choice scores and only the best `keep` groups stay in the
+ * choice (groups == 1 or keep == groups: all); the `top` largest choice scores are chosen; weights = s of the chosen
+ * / (their sum + 1e-20) * scale.  chosen int32 [rows, top], weights fp32 [rows, top]. */
+int swm_group_router(int32_t* chosen, float* weights, const float* logits, const float* correction, int64_t rows,
+                     int experts, int top, int groups, int keep, float scale, void* stream);
 
 /* Causal softmax attention of every new token over its sequence's paged keys with grouped query heads (query head
  * h reads key/value head h / (heads / kv_heads)): score = (q . k) * scale, then softcap * tanh(score / softcap) when
  * softcap > 0; position i sees j <= i (and i - j < window when window > 0); fp32 scores, weights and sums.
  * q fp32 [rows, heads * dim] (already rotated); caches [pages * page_size, kv_heads * dim | vdim] act_dtype;
  * gate (NULL: none) act_dtype [rows, heads * vdim] with row stride: the output is multiplied by sigmoid(gate);
- * out act_dtype [rows, heads * vdim]. */
+ * out act_dtype [rows, heads * vdim].  max_query_len: the most new tokens of any sequence (0: unknown); steps of
+ * few tokens per sequence split every sequence's keys over the waves of a workgroup. */
 int swm_capped_attention(void* out, const float* q, const void* key_cache, const void* value_cache,
                          const void* gate, int64_t gate_stride, const int32_t* block_tables, int table_width,
-                         const int32_t* q_start, const int32_t* ctx_len, int64_t rows, int num_seqs, int heads,
-                         int kv_heads, int dim, int vdim, int page_size, float scale, float softcap, int window,
-                         int act_dtype, void* stream);
+                         const int32_t* q_start, const int32_t* ctx_len, int64_t rows, int num_seqs,
+                         int max_query_len, int heads, int kv_heads, int dim, int vdim, int page_size, float scale,
+                         float softcap, int window, int act_dtype, void* stream);
 
 /* Linear attention with one decay per head:  S <- decay[h] S + k v^T;  o = S^T q, with q, k, v = silu of the given
  * projections (act_dtype, column ranges of one output with row stride in_stride; q, k [rows, heads * dim],

@@ -267,8 +267,8 @@ def test_group_router(E, top, groups, keep, dtype):
     correction = torch.randn(E, generator=g) * 0.6 - 0.5
     spec = {"experts": E, "top": top, "scale": 1.7, "groups": {"count": groups, "keep": keep}}
     for corr in (correction, None):
-        chosen, weights = ops().group_router(h.to(DEV), router.to(DEV), None if corr is None else corr.to(DEV), top, groups,
-                                             keep, 1.7)
+        logits = torch.matmul(h.to(DEV).float(), router.to(DEV).t())
+        chosen, weights = ops().group_router(logits, None if corr is None else corr.to(DEV), top, groups, keep, 1.7)
         w = {"router": router.double()}
         if corr is not None:
             w["correction"] = corr.double()

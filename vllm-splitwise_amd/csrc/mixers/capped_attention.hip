@@ -5,9 +5,10 @@
 //
 // Work split.  A tile is 32 query rows of ONE sequence and ONE key/value head: the R = heads / kv_heads query heads
 // of that group for 32 / R consecutive new tokens (row = token * R + head), so a decode step keeps all heads of a
-// group in one tile and a prompt shares every loaded key among R * tokens rows.  A workgroup of NW waves owns a
-// tile; wave w takes the 32-key tiles w, w + NW, ... of the visible keys with a running softmax of its own, and
-// the waves are joined through LDS in a fixed order (results do not depend on timing).
+// group in one tile and a prompt shares every loaded key among R * tokens rows.  In steps of prompt portions every
+// wave owns a tile and walks its keys alone.  In steps where no sequence brings more tokens than one tile holds (decode
+// steps) a workgroup of NW waves owns a tile; wave w takes the 32-key tiles w, w + NW, ... of the visible keys with a
+// running softmax of its own, and the waves are joined through LDS in a fixed order (results do not depend on timing).
 //
 // Matrix-core layouts (A [32 x 2], B [2 x 32], C [32 x 32] per instruction; lane l, half hl = l / 32):
 //   S^T = K Q^T : A = keys (row l % 32), B = queries (column l % 32); the two operands read the SAME coordinates in
@@ -83,49 +84,57 @@ __device__ __forceinline__ int find_query_tile(const int32_t* __restrict__ q_sta
   return 0;
 }
 
-// NVB: 32-channel blocks of the value size
+// NVB: 32-channel blocks of the value size.
+// split != 0 (steps in which no sequence brings more tokens than one tile holds, a decode step above all): a workgroup
+//   owns one tile and its waves share the keys out among them, joined through LDS (rows_used query rows are live).
+// split == 0: every wave owns a tile of its own and walks all of its keys; nothing is joined.
 template <typename T, int NVB>
-__global__ __launch_bounds__(256) void capped_attention_kernel(
+__global__ __launch_bounds__(512) void capped_attention_kernel(
     void* __restrict__ out, const float* __restrict__ q, const void* __restrict__ key_cache,
     const void* __restrict__ value_cache, const void* __restrict__ gate, int64_t gate_stride,
     const int32_t* __restrict__ block_tables, int table_width, const int32_t* __restrict__ q_start,
     const int32_t* __restrict__ ctx_len, int num_seqs, int heads, int kv_heads, int dim, int vdim, int page_size,
-    float scale, float softcap, int window, int tpt) {
+    float scale, float softcap, int window, int tpt, int split, int rows_used) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   const int R = heads / kv_heads;
   const int dblocks = (dim + 31) / 32;
   const int qstride = dblocks * 32 + 4;
   const int nw = blockDim.x >> 6;
   const int ostride = NVB * 32 + 1;
-  float* Qs = lds;                                           // [32][qstride], scaled queries, zero padded
-  float* Ml = Qs + kQT * qstride;                            // [nw][32][2]: running maximum and sum
-  float* Os = Ml + nw * kQT * 2;                             // [nw][32][ostride]
-
-  int seq, tok0;
-  const int ntok = find_query_tile(q_start, num_seqs, blockIdx.x, tpt, &seq, &tok0);
-  if (ntok == 0) return;                                     // uniform over the workgroup
-  const int g = blockIdx.y;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int qi = lane & 31, hl = lane >> 5;
-  const int64_t row0 = q_start[seq] + tok0;
-  const int ctx = ctx_len[seq];
+  // split: Qs [32][qstride] | Ml [nw][32][2] | Os [nw][rows_used][ostride];  else per wave one region for Qs, then Os
+  const int region = kQT * max(qstride, ostride);
+  float* Qs = split ? lds : lds + wave * region;
+  float* Ml = lds + kQT * qstride;
+  float* Os = split ? Ml + nw * kQT * 2 + wave * rows_used * ostride : Qs;
+
+  int seq = 0, tok0 = 0;
+  const int ntok = find_query_tile(q_start, num_seqs, split ? blockIdx.x : blockIdx.x * nw + wave, tpt, &seq, &tok0);
+  const bool live = ntok > 0;                                // uniform over the wave (over the workgroup when split)
+  const int g = blockIdx.y;
+  const int64_t row0 = live ? q_start[seq] + tok0 : 0;
+  const int ctx = live ? ctx_len[seq] : 0;
   const int32_t* table = block_tables + (int64_t)seq * table_width;
 
-  for (int e = threadIdx.x; e < kQT * dblocks * 32; e += blockDim.x) {
-    const int r = e / (dblocks * 32), c = e % (dblocks * 32);
-    const int tt = r / R, hh = r % R;
-    float v = 0.0f;
-    if (tt < ntok && c < dim) v = q[(row0 + tt) * (int64_t)heads * dim + (int64_t)(g * R + hh) * dim + c] * scale;
-    Qs[r * qstride + c] = v;
+  if (live) {
+    const int e0 = split ? threadIdx.x : lane, step = split ? blockDim.x : 64;
+    for (int e = e0; e < kQT * dblocks * 32; e += step) {
+      const int r = e / (dblocks * 32), c = e % (dblocks * 32);
+      const int tt = r / R, hh = r % R;
+      float v = 0.0f;
+      if (tt < ntok && c < dim) v = q[(row0 + tt) * (int64_t)heads * dim + (int64_t)(g * R + hh) * dim + c] * scale;
+      Qs[r * qstride + c] = v;
+    }
   }
   __syncthreads();
 
   const int first_pos = ctx + tok0, last_pos = ctx + tok0 + ntok - 1;
   // rows without a token behave like the tile's last token and are never stored
-  const int pos_q = first_pos + min(qi / R, ntok - 1);
+  const int pos_q = first_pos + min(qi / R, max(ntok - 1, 0));
   // keys below every row's window are skipped as whole tiles
   const int lowest = window > 0 ? max(0, first_pos - window + 1) : 0;
-  const int tile_lo = lowest / kQT, tile_hi = last_pos / kQT;
+  const int tile_lo = lowest / kQT, tile_hi = live ? last_pos / kQT : -1;
   const bool kvec = dim % 8 == 0;
 
   f32x16 o[NVB];
@@ -135,13 +144,20 @@ __global__ __launch_bounds__(256) void capped_attention_kernel(
     for (int r = 0; r < 16; ++r) o[b][r] = 0.0f;
   float m_run = -INFINITY, l_run = 0.0f;
 
-  for (int kt = tile_lo + wave; kt <= tile_hi; kt += nw) {
+  for (int kt = tile_lo + (split ? wave : 0); kt <= tile_hi; kt += (split ? nw : 1)) {
     const int k0 = kt * kQT;
     // ---- S^T = K Q^T
     const int key = k0 + qi;
     const bool key_ok = key <= last_pos;
     int64_t krow = 0;
     if (key_ok) krow = ((int64_t)table[key / page_size] * page_size + key % page_size) * kv_heads + g;
+    // rows of the values that this lane's weights meet: key (r, hl)
+    int64_t vrow[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int kj = k0 + 8 * (r / 4) + 4 * hl + (r % 4);
+      vrow[r] = kj <= last_pos ? ((int64_t)table[kj / page_size] * page_size + kj % page_size) * kv_heads + g : -1;
+    }
     f32x16 s;
 #pragma unroll
     for (int r = 0; r < 16; ++r) s[r] = 0.0f;
@@ -186,50 +202,72 @@ __global__ __launch_bounds__(256) void capped_attention_kernel(
     l_run = l_run * alpha + psum;
     m_run = m_new;
     // ---- O^T = alpha O^T + V^T P^T
-    int64_t vrow[16];
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int kj = k0 + 8 * (r / 4) + 4 * hl + (r % 4);
-      vrow[r] = kj <= last_pos ? ((int64_t)table[kj / page_size] * page_size + kj % page_size) * kv_heads + g : -1;
-    }
 #pragma unroll
     for (int b = 0; b < NVB; ++b) {
       const int vc = b * 32 + qi;
+      float vv[16];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        vv[r] = 0.0f;
+        if (vc < vdim && vrow[r] >= 0) vv[r] = ld<T>(value_cache, vrow[r] * vdim + vc);
+      }
 #pragma unroll
       for (int r = 0; r < 16; ++r) o[b][r] *= alpha;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        float vv = 0.0f;
-        if (vc < vdim && vrow[r] >= 0) vv = ld<T>(value_cache, vrow[r] * vdim + vc);
-        o[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv, p[r], o[b], 0, 0, 0);
-      }
+      for (int r = 0; r < 16; ++r) o[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv[r], p[r], o[b], 0, 0, 0);
     }
   }
 
-  // ---- join the waves
-  if (hl == 0) {
-    Ml[(wave * kQT + qi) * 2] = m_run;
-    Ml[(wave * kQT + qi) * 2 + 1] = l_run;
+  if (split) {
+    // ---- join the waves
+    if (!live) return;                                       // the whole workgroup
+    if (hl == 0) {
+      Ml[(wave * kQT + qi) * 2] = m_run;
+      Ml[(wave * kQT + qi) * 2 + 1] = l_run;
+    }
+    if (qi < rows_used) {
+#pragma unroll
+      for (int b = 0; b < NVB; ++b)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) Os[qi * ostride + b * 32 + 8 * (r / 4) + 4 * hl + (r % 4)] = o[b][r];
+    }
+    __syncthreads();
+    const float* Oall = Ml + nw * kQT * 2;
+    for (int e = threadIdx.x; e < rows_used * vdim; e += blockDim.x) {
+      const int r = e / vdim, c = e % vdim;
+      const int tt = r / R, hh = r % R;
+      if (tt >= ntok) continue;
+      float m_all = -INFINITY;
+      for (int w = 0; w < nw; ++w) m_all = fmaxf(m_all, Ml[(w * kQT + r) * 2]);
+      float num = 0.0f, den = 0.0f;
+      for (int w = 0; w < nw; ++w) {
+        const float f = expf(Ml[(w * kQT + r) * 2] - m_all);  // a wave that saw no key: exp(-inf) = 0
+        den += f * Ml[(w * kQT + r) * 2 + 1];
+        num += f * Oall[(w * rows_used + r) * ostride + c];
+      }
+      float v = num / den;
+      const int64_t col = (int64_t)(g * R + hh) * vdim + c;
+      if (gate != nullptr) v *= sigmoidf_(ld<T>(gate, (row0 + tt) * gate_stride + col));
+      st<T>(out, (row0 + tt) * (int64_t)heads * vdim + col, v);
+    }
+    return;
   }
-#pragma unroll
-  for (int b = 0; b < NVB; ++b)
-#pragma unroll
-    for (int r = 0; r < 16; ++r)
-      Os[(wave * kQT + qi) * ostride + b * 32 + 8 * (r / 4) + 4 * hl + (r % 4)] = o[b][r];
+  // ---- every wave for itself: turn O^T round through the wave's own LDS region (its queries are done with)
   __syncthreads();
-  for (int e = threadIdx.x; e < kQT * vdim; e += blockDim.x) {
+  if (live) {
+    const float inv = 1.0f / l_run;
+#pragma unroll
+    for (int b = 0; b < NVB; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) Os[qi * ostride + b * 32 + 8 * (r / 4) + 4 * hl + (r % 4)] = o[b][r] * inv;
+  }
+  __syncthreads();
+  if (!live) return;
+  for (int e = lane; e < kQT * vdim; e += 64) {
     const int r = e / vdim, c = e % vdim;
     const int tt = r / R, hh = r % R;
     if (tt >= ntok) continue;
-    float m_all = -INFINITY;
-    for (int w = 0; w < nw; ++w) m_all = fmaxf(m_all, Ml[(w * kQT + r) * 2]);
-    float num = 0.0f, den = 0.0f;
-    for (int w = 0; w < nw; ++w) {
-      const float f = expf(Ml[(w * kQT + r) * 2] - m_all);  // a wave that saw no key: exp(-inf) = 0
-      den += f * Ml[(w * kQT + r) * 2 + 1];
-      num += f * Os[(w * kQT + r) * ostride + c];
-    }
-    float v = num / den;
+    float v = Os[r * ostride + c];
     const int64_t col = (int64_t)(g * R + hh) * vdim + c;
     if (gate != nullptr) v *= sigmoidf_(ld<T>(gate, (row0 + tt) * gate_stride + col));
     st<T>(out, (row0 + tt) * (int64_t)heads * vdim + col, v);
@@ -239,16 +277,22 @@ __global__ __launch_bounds__(256) void capped_attention_kernel(
 template <typename T, int NVB>
 int launch_capped_attention(void* out, const float* q, const void* key_cache, const void* value_cache, const void* gate,
                             int64_t gate_stride, const int32_t* block_tables, int table_width, const int32_t* q_start,
-                            const int32_t* ctx_len, int64_t rows, int num_seqs, int heads, int kv_heads, int dim,
-                            int vdim, int page_size, float scale, float softcap, int window, hipStream_t stream) {
+                            const int32_t* ctx_len, int64_t rows, int num_seqs, int max_query_len, int heads,
+                            int kv_heads, int dim, int vdim, int page_size, float scale, float softcap, int window,
+                            hipStream_t stream) {
   const int R = heads / kv_heads;
   const int tpt = kQT / R;
-  const int dblocks = (dim + 31) / 32;
+  const int qstride = (dim + 31) / 32 * 32 + 4, ostride = NVB * 32 + 1;
+  const bool split = max_query_len > 0 && max_query_len <= tpt;
+  const int rows_used = split ? max_query_len * R : kQT;
   auto lds_bytes = [&](int nw) {
-    return (size_t)(kQT * (dblocks * 32 + 4) + nw * kQT * 2 + nw * kQT * (NVB * 32 + 1)) * sizeof(float);
+    const size_t floats = split ? (size_t)kQT * qstride + (size_t)nw * kQT * 2 + (size_t)nw * rows_used * ostride
+                                : (size_t)nw * kQT * std::max(qstride, ostride);
+    return floats * sizeof(float);
   };
-  int nw = 4;
-  while (nw > 1 && lds_bytes(nw) > 150 * 1024) nw >>= 1;
+  // two workgroups of a compute unit's 160 KB where the sizes allow it
+  int nw = split ? 8 : 4;
+  while (nw > 1 && lds_bytes(nw) > 72 * 1024) nw >>= 1;
   SW_CHECK_ARG(lds_bytes(nw) <= 160 * 1024, "capped_attention: key size %d with value size %d needs too much LDS", dim,
                vdim);
   auto kernel = capped_attention_kernel<T, NVB>;
@@ -258,10 +302,11 @@ int launch_capped_attention(void* out, const float* q, const void* key_cache, co
                                      (int)lds_bytes(nw)));
     allowed = lds_bytes(nw);
   }
-  const dim3 grid((unsigned)((rows + tpt - 1) / tpt + num_seqs), (unsigned)kv_heads);
+  const int64_t tiles = split ? num_seqs : (rows + tpt - 1) / tpt + num_seqs;
+  const dim3 grid((unsigned)(split ? tiles : (tiles + nw - 1) / nw), (unsigned)kv_heads);
   hipLaunchKernelGGL(kernel, grid, dim3(64 * nw), lds_bytes(nw), stream, out, q, key_cache, value_cache, gate,
                      gate_stride, block_tables, table_width, q_start, ctx_len, num_seqs, heads, kv_heads, dim, vdim,
-                     page_size, scale, softcap, window, tpt);
+                     page_size, scale, softcap, window, tpt, split ? 1 : 0, rows_used);
   SW_CHECK_LAUNCH();
   return SW_OK;
 }
@@ -271,7 +316,7 @@ int launch_capped_attention(void* out, const float* q, const void* key_cache, co
 extern "C" int swm_capped_attention(void* out, const float* q, const void* key_cache, const void* value_cache,
                                     const void* gate, int64_t gate_stride, const int32_t* block_tables,
                                     int table_width, const int32_t* q_start, const int32_t* ctx_len, int64_t rows,
-                                    int num_seqs, int heads, int kv_heads, int dim, int vdim, int page_size,
+                                    int num_seqs, int max_query_len, int heads, int kv_heads, int dim, int vdim, int page_size,
                                     float scale, float softcap, int window, int act_dtype, void* stream) {
   using namespace swm;
   if (rows == 0 || num_seqs == 0) return SW_OK;
@@ -287,8 +332,8 @@ extern "C" int swm_capped_attention(void* out, const float* q, const void* key_c
   case N:                                                                                                               \
     SWM_DISPATCH_ACT(act_dtype, return (launch_capped_attention<T, N>(                                                  \
                                     out, q, key_cache, value_cache, gate, gate_stride, block_tables, table_width,       \
-                                    q_start, ctx_len, rows, num_seqs, heads, kv_heads, dim, vdim, page_size, scale,     \
-                                    softcap, window, s)););                                                             \
+                                    q_start, ctx_len, rows, num_seqs, max_query_len, heads, kv_heads, dim, vdim,        \
+                                    page_size, scale, softcap, window, s)););                                                             \
     break;
   switch (nvb) {
     SWM_CAPPED_CASE(1)

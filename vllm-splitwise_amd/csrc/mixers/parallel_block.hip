@@ -4,8 +4,8 @@
 //   * clamped_glu / relu2: activations between the library GEMMs of a feed-forward;
 //   * rope_cache: partial rotary embedding on neighbouring pairs from a table of per-pair frequencies (angles
 //     from fp32 positions), rotated queries out in fp32, rotated keys and values into the paged cache;
-//   * group_router: sigmoid router with a selection bias, a limit to the best groups of experts and weights
-//     normalised over the chosen ones.
+//   * group_router: the choice of a sigmoid router from its fp32 logits: a selection bias, a limit to the best
+//     groups of experts and weights normalised over the chosen ones.
 // All arithmetic is fp32; activations are read and written in the model's dtype.
 #include "mixers_common.cuh"
 
@@ -118,31 +118,27 @@ __global__ __launch_bounds__(kPbThreads) void rope_cache_kernel(
     st<T>(value_cache, slot * (int64_t)kv_heads * vdim + e, ld<T>(v, row + e));
 }
 
-// one wave per row: the router's products over the lanes, the choice by lane 0
+// one wave per row: scores by the lanes, the choice by lane 0 (a few hundred LDS reads for the usual sizes)
 constexpr int kMaxRouterExperts = 256;
 
-template <typename T>
 __global__ __launch_bounds__(256) void group_router_kernel(
-    int32_t* __restrict__ chosen, float* __restrict__ weights, const void* __restrict__ h, int64_t h_stride,
-    const float* __restrict__ router, const float* __restrict__ correction, int64_t rows, int width, int experts,
-    int top, int groups, int keep, float scale) {
+    int32_t* __restrict__ chosen, float* __restrict__ weights, const float* __restrict__ logits,
+    const float* __restrict__ correction, int64_t rows, int experts, int top, int groups, int keep, float scale) {
   __shared__ float s_score[4][kMaxRouterExperts];
   __shared__ float s_choice[4][kMaxRouterExperts];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int64_t t = (int64_t)blockIdx.x * 4 + wave;
-  if (t >= rows) return;                                   // uniform over the wave; no workgroup barrier below
+  const bool live = t < rows;
   float* score = s_score[wave];
   float* choice = s_choice[wave];
-  for (int e = 0; e < experts; ++e) {
-    float z = 0.0f;
-    for (int i = lane; i < width; i += 64) z += router[(int64_t)e * width + i] * ld<T>(h, t * h_stride + i);
-    z = sw::wave_sum(z);
-    if (lane == 0) {
-      const float s = sigmoidf_(z);
+  if (live)
+    for (int e = lane; e < experts; e += 64) {
+      const float s = sigmoidf_(logits[t * experts + e]);
       score[e] = s;
       choice[e] = s + (correction != nullptr ? correction[e] : 0.0f);
     }
-  }
+  __syncthreads();
+  if (!live) return;
   if (lane != 0) return;
   const float kOut = -INFINITY;
   if (groups > 1 && keep < groups) {
@@ -247,20 +243,17 @@ int swm_rope_cache(float* q_out, const void* q, const void* k, const void* v, in
   return SW_OK;
 }
 
-int swm_group_router(int32_t* chosen, float* weights, const void* h, int64_t h_stride, const float* router,
-                     const float* correction, int64_t rows, int width, int experts, int top, int groups, int keep,
-                     float scale, int act_dtype, void* stream) {
+int swm_group_router(int32_t* chosen, float* weights, const float* logits, const float* correction, int64_t rows,
+                     int experts, int top, int groups, int keep, float scale, void* stream) {
   using namespace swm;
   if (rows == 0) return SW_OK;
-  SW_CHECK_ARG(act_ok(act_dtype), "group_router: unsupported dtype %d", act_dtype);
-  SW_CHECK_ARG(experts > 0 && experts <= kMaxRouterExperts && top > 0 && top <= experts && width > 0,
+  SW_CHECK_ARG(experts > 0 && experts <= kMaxRouterExperts && top > 0 && top <= experts,
                "group_router: %d experts (1..%d supported), top %d", experts, kMaxRouterExperts, top);
   SW_CHECK_ARG(groups >= 1 && keep >= 1 && keep <= groups && experts % groups == 0 &&
                    (int64_t)keep * (experts / groups) >= top,
                "group_router: %d groups, %d kept, %d experts, top %d", groups, keep, experts, top);
-  SWM_DISPATCH_ACT(act_dtype, hipLaunchKernelGGL(group_router_kernel<T>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
-                                                 static_cast<hipStream_t>(stream), chosen, weights, h, h_stride, router,
-                                                 correction, rows, width, experts, top, groups, keep, scale););
+  hipLaunchKernelGGL(group_router_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     chosen, weights, logits, correction, rows, experts, top, groups, keep, scale);
   SW_CHECK_LAUNCH();
   return SW_OK;
 }

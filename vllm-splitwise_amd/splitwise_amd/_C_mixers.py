@@ -43,8 +43,9 @@ _SIGNATURES = {
     "swm_clamped_glu": [_p, _p, _l, _l, _i, _f, _f, _f, _i, _p],
     "swm_relu2": [_p, _p, _l, _l, _i, _i, _p],
     "swm_rope_cache": [_p, _p, _p, _p, _l, _p, _p, _i, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p],
-    "swm_group_router": [_p, _p, _p, _l, _p, _p, _l, _i, _i, _i, _i, _i, _f, _i, _p],
-    "swm_capped_attention": [_p, _p, _p, _p, _p, _l, _p, _i, _p, _p, _l, _i, _i, _i, _i, _i, _i, _f, _f, _i, _i, _p],
+    "swm_group_router": [_p, _p, _p, _p, _l, _i, _i, _i, _i, _f, _p],
+    "swm_capped_attention": [_p, _p, _p, _p, _p, _l, _p, _i, _p, _p, _l, _i, _i, _i, _i, _i, _i, _i, _f, _f, _i, _i,
+                             _p],
     "swm_lightning": [_p, _p, _p, _p, _l, _p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p],
 }
 ACT_GELU, ACT_RELU2 = 0, 1
@@ -449,23 +450,21 @@ def rope_cache(q_out: torch.Tensor, q: torch.Tensor, k: Optional[torch.Tensor], 
             kv_heads, dim, vdim, _act(q), _stream(q)))
 
 
-def group_router(h: torch.Tensor, router: torch.Tensor, correction: Optional[torch.Tensor], top: int, groups: int,
-                 keep: int, scale: float):
-    """-> (chosen int32 [rows, top], weights fp32 [rows, top])."""
-    _dev(h, router, correction)
-    _f32c(router, "router")
-    rows, width = h.shape
-    experts = router.shape[0]
-    _need(router.shape == (experts, width), "group_router: router shape")
+def group_router(logits: torch.Tensor, correction: Optional[torch.Tensor], top: int, groups: int, keep: int,
+                 scale: float):
+    """logits fp32 [rows, experts] -> (chosen int32 [rows, top], weights fp32 [rows, top])."""
+    _dev(logits, correction)
+    _f32c(logits, "logits")
+    rows, experts = logits.shape
     if correction is not None:
         _f32c(correction, "correction")
         _need(correction.numel() == experts, "group_router: correction")
-    chosen = torch.empty(rows, top, dtype=torch.int32, device=h.device)
-    weights = torch.empty(rows, top, dtype=torch.float32, device=h.device)
-    with _on_device_of(h):
-        _check(load_library().swm_group_router(chosen.data_ptr(), weights.data_ptr(), h.data_ptr(), _rows(h, "h"),
-                                               router.data_ptr(), _opt_ptr(correction), rows, width, experts, top,
-                                               groups, keep, scale, _act(h), _stream(h)))
+    chosen = torch.empty(rows, top, dtype=torch.int32, device=logits.device)
+    weights = torch.empty(rows, top, dtype=torch.float32, device=logits.device)
+    with _on_device_of(logits):
+        _check(load_library().swm_group_router(chosen.data_ptr(), weights.data_ptr(), logits.data_ptr(),
+                                               _opt_ptr(correction), rows, experts, top, groups, keep, scale,
+                                               _stream(logits)))
     return chosen, weights
 
 
@@ -494,8 +493,8 @@ def capped_attention(out: torch.Tensor, q: torch.Tensor, key_cache: torch.Tensor
         _check(load_library().swm_capped_attention(
             out.data_ptr(), q.data_ptr(), key_cache.data_ptr(), value_cache.data_ptr(), _opt_ptr(gate),
             0 if gate is None else _rows(gate, "gate"), tables.data_ptr(), tables.shape[1], batch.q_start.data_ptr(),
-            batch.ctx_len.data_ptr(), rows, n, heads, kv_heads, dim, vdim, key_cache.shape[1], scale, softcap, window,
-            _act(out), _stream(q)))
+            batch.ctx_len.data_ptr(), rows, n, int(getattr(batch, "max_query_len", 0) or 0), heads, kv_heads, dim, vdim,
+            key_cache.shape[1], scale, softcap, window, _act(out), _stream(q)))
 
 
 def lightning(out: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor,

@@ -375,10 +375,10 @@ def kernel_table_lapilorn(width: int = 2048, heads: int = 16, kv_heads: int = 4,
         hin = torch.randn(T, width, device=dev).to(bf)
         router = torch.randn(experts, width, device=dev) * width ** -0.5
         corr = torch.randn(experts, device=dev) * 0.1
-        t = _time(lambda: _C.mixer_ops.group_router(hin, router, corr, top, 4, 2, 2.5))
-        rows.append(_row("group_router (fp32)", phase, t, T * width * 2 + experts * width * 4 + T * top * 8,
+        t = _time(lambda: _C.mixer_ops.group_router(torch.matmul(hin.float(), router.t()), corr, top, 4, 2, 2.5))
+        rows.append(_row("router: fp32 GEMM + group_router", phase, t, T * width * 2 + experts * width * 4 + T * top * 8,
                          2.0 * T * experts * width, VALU_F32))
-        chosen, weights = _C.mixer_ops.group_router(hin, router, corr, top, 4, 2, 2.5)
+        chosen, weights = _C.mixer_ops.group_router(torch.matmul(hin.float(), router.t()), corr, top, 4, 2, 2.5)
         from ..model_executor.layers.moe import group_pairs_by_expert
         order, start = group_pairs_by_expert(chosen, experts)
         up = torch.randn(experts, ff, width, device=dev).to(bf) * 0.02

@@ -97,7 +97,9 @@ class GroupRoutedExperts(nn.Module):
 
     def forward(self, h: torch.Tensor) -> Tuple[Optional[torch.Tensor], torch.Tensor]:
         """-> (shared expert's output in h's dtype or None, routed experts' weighted sum in fp32)."""
-        chosen, weights = _C.mixer_ops.group_router(h, self.router.data, self.correction.data, self.top, self.groups,
+        # fp32 products with the fp32 router (the library's GEMM; no reduced-precision matrix mode is switched on)
+        logits = torch.matmul(h.float(), self.router.data.t())
+        chosen, weights = _C.mixer_ops.group_router(logits, self.correction.data, self.top, self.groups,
                                                     self.keep_groups, self.scale)
         order, start = group_pairs_by_expert(chosen, self.num_experts)
         out = torch.zeros(h.shape[0], self.width, dtype=torch.float32, device=h.device)
