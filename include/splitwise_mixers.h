@@ -190,10 +190,15 @@ int swm_capped_attention(void* out, const float* q, const void* key_cache, const
 
 /* Linear attention with one decay per head:  S <- decay[h] S + k v^T;  o = S^T q, with q, k, v = silu of the given
  * projections (act_dtype, column ranges of one output with row stride in_stride; q, k [rows, heads * dim],
- * v [rows, heads * vdim]); decay fp32 [heads]; state fp32 [slots, heads, dim, vdim]; out fp32 [rows, heads * vdim]. */
+ * v [rows, heads * vdim]); decay fp32 [heads]; state fp32 [slots, heads, dim, vdim]; out fp32 [rows, heads * vdim].
+ * max_query_len: the most new tokens of any sequence (0: unknown).  Long runs are cut into segments that run side by
+ * side and are joined by a scan over their end states; `workspace` then holds swm_lightning_workspace_floats() floats
+ * (0: the step has no long run; NULL: never cut). */
+int64_t swm_lightning_workspace_floats(int64_t rows, int num_seqs, int max_query_len, int heads, int dim, int vdim);
 int swm_lightning(float* out, const void* q, const void* k, const void* v, int64_t in_stride, const float* decay,
                   float* state, const int32_t* q_start, const int32_t* ctx_len, const int32_t* state_slot, int64_t rows,
-                  int num_seqs, int heads, int dim, int vdim, int act_dtype, void* stream);
+                  int num_seqs, int max_query_len, int heads, int dim, int vdim, float* workspace, int act_dtype,
+                  void* stream);
 
 #ifdef __cplusplus
 }

@@ -227,17 +227,18 @@ def _run_lightning(proj, sizes, decay, state, steps, H, d, dv):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_lightning_recurrence(H, d, dv, decay, dtype):
     """Two sequences interleaved over three state slots that held other sequences before: whole chunks, chunk
-    borders (31, 32, 33 tokens), portions of one and two tokens, a first portion of one token, and 70 tokens
-    decoded one by one; against the recurrence run token by token in double precision."""
+    borders (31, 32, 33 tokens), portions of one and two tokens, a first portion of one token, a run long enough
+    to be cut into segments that run side by side (from a carried state, beside a single token of the other
+    sequence), and 70 tokens decoded one by one; against the recurrence run token by token in double precision."""
     g = torch.Generator().manual_seed(H * 100 + d)
     nk, nv = H * d, H * dv
-    lens = {"a": 260, "b": 139}
+    lens = {"a": 640, "b": 139}
     proj = {s: (torch.randn(n, 2 * nk + nv + 3, generator=g) * 1.2).to(dtype) for s, n in lens.items()}
     state = torch.full((3, H, d, dv), float("nan"), dtype=torch.float32, device=DEV)     # slots are never cleared
     dec = torch.tensor(decay, dtype=torch.float32, device=DEV)
     steps = [[("a", 0, 1, 2)], [("a", 1, 31, 2), ("b", 0, 33, 0)], [("b", 33, 2, 0), ("a", 32, 32, 2)],
-             [("a", 64, 33, 2)], [("a", 97, 2, 2), ("b", 35, 64, 0)], [("a", 99, 91, 2), ("b", 99, 1, 0)]]
-    steps += [[("a", 190 + i, 1, 2)] + ([("b", 100 + i, 1, 0)] if i < 39 else []) for i in range(70)]
+             [("a", 64, 33, 2)], [("a", 97, 2, 2), ("b", 35, 64, 0)], [("a", 99, 471, 2), ("b", 99, 1, 0)]]
+    steps += [[("a", 570 + i, 1, 2)] + ([("b", 100 + i, 1, 0)] if i < 39 else []) for i in range(70)]
     outs = _run_lightning(proj, (nk, nv), dec, state, steps, H, d, dv)
     silu = torch.nn.functional.silu
     final = {}
@@ -250,8 +251,10 @@ def test_lightning_recurrence(H, d, dv, decay, dtype):
     assert (state[2].cpu().double() - final["a"]).abs().max() < 2e-5 * final["a"].abs().max()
     assert (state[0].cpu().double() - final["b"]).abs().max() < 2e-5 * final["b"].abs().max()
     # a new sequence in a used slot starts from nothing, and one long run equals the portions
-    whole = _run_lightning({"b": proj["b"]}, (nk, nv), dec, state, [[("b", 0, lens["b"], 2)]], H, d, dv)
-    assert (whole["b"] - outs["b"]).abs().max() < 2e-5 * outs["b"].abs().max()
+    whole = _run_lightning(proj, (nk, nv), dec, state, [[("b", 0, lens["b"], 2), ("a", 0, lens["a"], 1)]], H, d, dv)
+    for s in lens:
+        assert (whole[s] - outs[s]).abs().max() < 2e-5 * outs[s].abs().max()
+    assert (state[1].cpu().double() - final["a"]).abs().max() < 2e-5 * final["a"].abs().max()
 
 
 @pytest.mark.parametrize("E,top,groups,keep", [(8, 3, 4, 3), (6, 2, 3, 2), (5, 1, 1, 1), (12, 4, 4, 2), (4, 2, 4, 3), (16, 6, 2, 1),

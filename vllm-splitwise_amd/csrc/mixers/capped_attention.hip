@@ -25,81 +25,95 @@ using f32x16 = __attribute__((ext_vector_type(16))) float;
 
 constexpr int kQT = 32;               // query rows and keys per tile
 
-// 16 consecutive coordinates [c0, c0 + 16) of a row of `size` coordinates, zeros beyond; `vec`: size % 8 == 0
-template <typename T>
-__device__ __forceinline__ void load_run16(float (&out)[16], const void* base, int64_t row_off, int c0, int size,
-                                           bool row_ok, bool vec);
-template <>
-__device__ __forceinline__ void load_run16<float>(float (&out)[16], const void* base, int64_t row_off, int c0,
-                                                  int size, bool row_ok, bool vec) {
-  const float* p = static_cast<const float*>(base) + row_off;
-  if (vec) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (row_ok && c0 + 4 * j + 4 <= size) v = *reinterpret_cast<const float4*>(p + c0 + 4 * j);
-      out[4 * j] = v.x; out[4 * j + 1] = v.y; out[4 * j + 2] = v.z; out[4 * j + 3] = v.w;
-    }
-  } else {
-#pragma unroll
-    for (int j = 0; j < 16; ++j) out[j] = (row_ok && c0 + j < size) ? p[c0 + j] : 0.0f;
+// N consecutive elements of a cache row as they are stored (bf16 two to a register), widened where they are used:
+// all loads of a key tile are issued before its first product, so their latencies overlap.
+template <typename T, int N> struct Raw;
+template <int N> struct Raw<float, N> {
+  float f[N];
+  __device__ __forceinline__ float get(int j) const { return f[j]; }
+};
+template <int N> struct Raw<bf16_t, N> {
+  uint32_t w[(N + 1) / 2];
+  __device__ __forceinline__ float get(int j) const {
+    return __uint_as_float((j & 1) ? (w[j / 2] & 0xffff0000u) : (w[j / 2] << 16));
   }
-}
-template <>
-__device__ __forceinline__ void load_run16<bf16_t>(float (&out)[16], const void* base, int64_t row_off, int c0,
-                                                   int size, bool row_ok, bool vec) {
-  const uint16_t* p = static_cast<const uint16_t*>(base) + row_off;
+};
+
+// elements [c0, c0 + N) of the row at `row_off` (elements) of `size` coordinates, zeros beyond or when !ok;
+// `vec`: N is a power of two, N <= 16 bytes' worth per load piece, and size, row_off are multiples of N
+template <int N>
+__device__ __forceinline__ void load_raw(Raw<float, N>& out, const void* base, int64_t row_off, int c0, int size,
+                                         bool ok, bool vec) {
+  const float* p = static_cast<const float*>(base) + row_off + c0;
   if (vec) {
+    if constexpr (N % 4 == 0) {
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      uint4 v = make_uint4(0u, 0u, 0u, 0u);
-      if (row_ok && c0 + 8 * j + 8 <= size) v = *reinterpret_cast<const uint4*>(p + c0 + 8 * j);
-      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        out[8 * j + 2 * e] = __uint_as_float(w[e] << 16);
-        out[8 * j + 2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
+      for (int j = 0; j < N / 4; ++j) {
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (ok && c0 + 4 * j < size) v = *reinterpret_cast<const float4*>(p + 4 * j);
+        out.f[4 * j] = v.x; out.f[4 * j + 1] = v.y; out.f[4 * j + 2] = v.z; out.f[4 * j + 3] = v.w;
       }
+    } else if constexpr (N == 2) {
+      float2 v = make_float2(0.f, 0.f);
+      if (ok && c0 < size) v = *reinterpret_cast<const float2*>(p);
+      out.f[0] = v.x; out.f[1] = v.y;
+    } else {
+      out.f[0] = (ok && c0 < size) ? p[0] : 0.0f;
     }
   } else {
 #pragma unroll
-    for (int j = 0; j < 16; ++j) out[j] = (row_ok && c0 + j < size) ? sw::bf16_bits_to_float(p[c0 + j]) : 0.0f;
+    for (int j = 0; j < N; ++j) out.f[j] = (ok && c0 + j < size) ? p[j] : 0.0f;
   }
 }
-
-// -> sequence and first new token of tile `tile` when every sequence's new tokens are cut into runs of `tpt`;
-//    returns the tokens in the tile (0: no such tile)
-__device__ __forceinline__ int find_query_tile(const int32_t* __restrict__ q_start, int num_seqs, int tile, int tpt,
-                                               int* seq, int* tok0) {
-  for (int s = 0; s < num_seqs; ++s) {
-    const int n = q_start[s + 1] - q_start[s];
-    const int tiles = (n + tpt - 1) / tpt;
-    if (tile < tiles) {
-      *seq = s;
-      *tok0 = tile * tpt;
-      return min(tpt, n - tile * tpt);
+template <int N>
+__device__ __forceinline__ void load_raw(Raw<bf16_t, N>& out, const void* base, int64_t row_off, int c0, int size,
+                                         bool ok, bool vec) {
+  const uint16_t* p = static_cast<const uint16_t*>(base) + row_off + c0;
+  if (vec && N % 2 == 0) {
+    if constexpr (N % 8 == 0) {
+#pragma unroll
+      for (int j = 0; j < N / 8; ++j) {
+        uint4 v = make_uint4(0u, 0u, 0u, 0u);
+        if (ok && c0 + 8 * j < size) v = *reinterpret_cast<const uint4*>(p + 8 * j);
+        out.w[4 * j] = v.x; out.w[4 * j + 1] = v.y; out.w[4 * j + 2] = v.z; out.w[4 * j + 3] = v.w;
+      }
+    } else if constexpr (N == 4) {
+      uint2 v = make_uint2(0u, 0u);
+      if (ok && c0 < size) v = *reinterpret_cast<const uint2*>(p);
+      out.w[0] = v.x; out.w[1] = v.y;
+    } else if constexpr (N == 2) {
+      out.w[0] = (ok && c0 < size) ? *reinterpret_cast<const uint32_t*>(p) : 0u;
     }
-    tile -= tiles;
+  } else {
+#pragma unroll
+    for (int j = 0; j < (N + 1) / 2; ++j) {
+      const uint32_t lo = (ok && c0 + 2 * j < size) ? p[2 * j] : 0u;
+      const uint32_t hi = (2 * j + 1 < N && ok && c0 + 2 * j + 1 < size) ? p[2 * j + 1] : 0u;
+      out.w[j] = lo | (hi << 16);
+    }
   }
-  return 0;
 }
 
-// NVB: 32-channel blocks of the value size.
+constexpr bool is_pow2(int n) { return n > 0 && (n & (n - 1)) == 0; }
+
+// NB: the larger of the numbers of 32-coordinate blocks of the key size and of the value size.  A lane's value
+// channels are NB neighbours (channel = NB * (l % 32) + block), so one load brings a key's values for all blocks.
 // split != 0 (steps in which no sequence brings more tokens than one tile holds, a decode step above all): a workgroup
 //   owns one tile and its waves share the keys out among them, joined through LDS (rows_used query rows are live).
 // split == 0: every wave owns a tile of its own and walks all of its keys; nothing is joined.
-template <typename T, int NVB>
+template <typename T, int NB>
 __global__ __launch_bounds__(512) void capped_attention_kernel(
     void* __restrict__ out, const float* __restrict__ q, const void* __restrict__ key_cache,
     const void* __restrict__ value_cache, const void* __restrict__ gate, int64_t gate_stride,
     const int32_t* __restrict__ block_tables, int table_width, const int32_t* __restrict__ q_start,
     const int32_t* __restrict__ ctx_len, int num_seqs, int heads, int kv_heads, int dim, int vdim, int page_size,
-    float scale, float softcap, int window, int tpt, int split, int rows_used) {
+    float scale, float softcap, int window, int tpt, int split, int rows_used, int page_shift) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   const int R = heads / kv_heads;
   const int dblocks = (dim + 31) / 32;
   const int qstride = dblocks * 32 + 4;
   const int nw = blockDim.x >> 6;
+  constexpr int NVB = NB;
   const int ostride = NVB * 32 + 1;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int qi = lane & 31, hl = lane >> 5;
@@ -136,6 +150,7 @@ __global__ __launch_bounds__(512) void capped_attention_kernel(
   const int lowest = window > 0 ? max(0, first_pos - window + 1) : 0;
   const int tile_lo = lowest / kQT, tile_hi = live ? last_pos / kQT : -1;
   const bool kvec = dim % 8 == 0;
+  const float inv_cap = softcap > 0.0f ? 1.0f / softcap : 0.0f;
 
   f32x16 o[NVB];
 #pragma unroll
@@ -144,35 +159,63 @@ __global__ __launch_bounds__(512) void capped_attention_kernel(
     for (int r = 0; r < 16; ++r) o[b][r] = 0.0f;
   float m_run = -INFINITY, l_run = 0.0f;
 
-  for (int kt = tile_lo + (split ? wave : 0); kt <= tile_hi; kt += (split ? nw : 1)) {
-    const int k0 = kt * kQT;
-    // ---- S^T = K Q^T
+  const bool vvec = is_pow2(NB) && vdim % NB == 0;
+  const int kstep = split ? nw : 1;
+  // cache slot of key k0 + qi of a tile (-1: beyond the tile's last key)
+  auto slot_of = [&](int k0) {
     const int key = k0 + qi;
-    const bool key_ok = key <= last_pos;
-    int64_t krow = 0;
-    if (key_ok) krow = ((int64_t)table[key / page_size] * page_size + key % page_size) * kv_heads + g;
-    // rows of the values that this lane's weights meet: key (r, hl)
-    int64_t vrow[16];
+    if (key > last_pos) return -1;
+    if (page_shift >= 0) return (table[key >> page_shift] << page_shift) + (key & (page_size - 1));
+    return table[key / page_size] * page_size + key % page_size;
+  };
+  // all loads of one key tile: this lane's key row (runs of 16 per block) and the values of keys (r, hl)
+  auto issue = [&](int slot, Raw<T, 16> (&kraw)[NB], Raw<T, NB> (&vraw)[16]) {
+    const int64_t krow = ((int64_t)max(slot, 0) * kv_heads + g) * dim;
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+      if (b < dblocks) load_raw(kraw[b], key_cache, krow, b * 32 + hl * 16, dim, slot >= 0, kvec);
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      const int kj = k0 + 8 * (r / 4) + 4 * hl + (r % 4);
-      vrow[r] = kj <= last_pos ? ((int64_t)table[kj / page_size] * page_size + kj % page_size) * kv_heads + g : -1;
+      const int vslot = __shfl(slot, 8 * (r / 4) + 4 * hl + (r % 4), 64);
+      load_raw(vraw[r], value_cache, ((int64_t)max(vslot, 0) * kv_heads + g) * vdim, qi * NB, vdim, vslot >= 0, vvec);
     }
+  };
+  // small heads in a 16-bit cache: the next tile's loads are in flight while this tile's products run (two register
+  // sets); otherwise there are registers for one set only, and the next tile is loaded after the products
+  constexpr bool kAhead = sizeof(typename Conv<T>::store_t) == 2 && NB <= 2;
+  int kt = tile_lo + (split ? wave : 0);
+  Raw<T, 16> kraw[NB];
+  Raw<T, NB> vraw[16];
+  int slot_next = -1;
+  if (kt <= tile_hi) {
+    issue(slot_of(kt * kQT), kraw, vraw);
+    if (kt + kstep <= tile_hi) slot_next = slot_of((kt + kstep) * kQT);
+  }
+  for (; kt <= tile_hi; kt += kstep) {
+    const int k0 = kt * kQT;
+    Raw<T, 16> kraw2[NB];
+    Raw<T, NB> vraw2[16];
+    int slot_next2 = -1;
+    if (kAhead) {
+      if (kt + kstep <= tile_hi) issue(slot_next, kraw2, vraw2);
+      if (kt + 2 * kstep <= tile_hi) slot_next2 = slot_of((kt + 2 * kstep) * kQT);
+    }
+    // ---- S^T = K Q^T
     f32x16 s;
 #pragma unroll
     for (int r = 0; r < 16; ++r) s[r] = 0.0f;
-    for (int db = 0; db < dblocks; ++db) {
-      const int c0 = db * 32 + hl * 16;
-      float kf[16];
-      load_run16<T>(kf, key_cache, krow * dim, c0, dim, key_ok, kvec);
-      const float4* qp = reinterpret_cast<const float4*>(Qs + qi * qstride + c0);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const float4 qv = qp[j];
-        s = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[4 * j], qv.x, s, 0, 0, 0);
-        s = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[4 * j + 1], qv.y, s, 0, 0, 0);
-        s = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[4 * j + 2], qv.z, s, 0, 0, 0);
-        s = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[4 * j + 3], qv.w, s, 0, 0, 0);
+    for (int b = 0; b < NB; ++b) {
+      if (b < dblocks) {
+        const float4* qp = reinterpret_cast<const float4*>(Qs + qi * qstride + b * 32 + hl * 16);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float4 qv = qp[j];
+          s = __builtin_amdgcn_mfma_f32_32x32x2f32(kraw[b].get(4 * j), qv.x, s, 0, 0, 0);
+          s = __builtin_amdgcn_mfma_f32_32x32x2f32(kraw[b].get(4 * j + 1), qv.y, s, 0, 0, 0);
+          s = __builtin_amdgcn_mfma_f32_32x32x2f32(kraw[b].get(4 * j + 2), qv.z, s, 0, 0, 0);
+          s = __builtin_amdgcn_mfma_f32_32x32x2f32(kraw[b].get(4 * j + 3), qv.w, s, 0, 0, 0);
+        }
       }
     }
     // ---- cap, mask, running softmax (this lane: query qi, keys (r, hl))
@@ -182,7 +225,7 @@ __global__ __launch_bounds__(512) void capped_attention_kernel(
     for (int r = 0; r < 16; ++r) {
       const int kj = k0 + 8 * (r / 4) + 4 * hl + (r % 4);
       float v = s[r];
-      if (softcap > 0.0f) v = softcap * tanhf(v / softcap);
+      if (softcap > 0.0f) v = softcap * fast_tanhf_(v * inv_cap);
       const bool seen = kj <= pos_q && (window <= 0 || pos_q - kj < window);
       v = seen ? v : -INFINITY;
       p[r] = v;
@@ -191,11 +234,11 @@ __global__ __launch_bounds__(512) void capped_attention_kernel(
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
     const float m_new = fmaxf(m_run, tmax);
     const float m_use = m_new == -INFINITY ? 0.0f : m_new;
-    const float alpha = expf(m_run - m_use);                 // 0 while nothing has been seen
+    const float alpha = fast_expf_(m_run - m_use);           // 0 while nothing has been seen
     float psum = 0.0f;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      p[r] = expf(p[r] - m_use);
+      p[r] = fast_expf_(p[r] - m_use);
       psum += p[r];
     }
     psum += __shfl_xor(psum, 32, 64);
@@ -203,18 +246,23 @@ __global__ __launch_bounds__(512) void capped_attention_kernel(
     m_run = m_new;
     // ---- O^T = alpha O^T + V^T P^T
 #pragma unroll
-    for (int b = 0; b < NVB; ++b) {
-      const int vc = b * 32 + qi;
-      float vv[16];
+    for (int b = 0; b < NB; ++b) {
+      if (b < vdim) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        vv[r] = 0.0f;
-        if (vc < vdim && vrow[r] >= 0) vv[r] = ld<T>(value_cache, vrow[r] * vdim + vc);
+        for (int r = 0; r < 16; ++r) o[b][r] *= alpha;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(vraw[r].get(b), p[r], o[b], 0, 0, 0);
       }
+    }
+    if (kAhead) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) o[b][r] *= alpha;
+      for (int b = 0; b < NB; ++b) kraw[b] = kraw2[b];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) o[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv[r], p[r], o[b], 0, 0, 0);
+      for (int r = 0; r < 16; ++r) vraw[r] = vraw2[r];
+      slot_next = slot_next2;
+    } else if (kt + kstep <= tile_hi) {
+      issue(slot_next, kraw, vraw);
+      slot_next = kt + 2 * kstep <= tile_hi ? slot_of((kt + 2 * kstep) * kQT) : -1;
     }
   }
 
@@ -229,7 +277,7 @@ __global__ __launch_bounds__(512) void capped_attention_kernel(
 #pragma unroll
       for (int b = 0; b < NVB; ++b)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) Os[qi * ostride + b * 32 + 8 * (r / 4) + 4 * hl + (r % 4)] = o[b][r];
+        for (int r = 0; r < 16; ++r) Os[qi * ostride + (8 * (r / 4) + 4 * hl + (r % 4)) * NB + b] = o[b][r];
     }
     __syncthreads();
     const float* Oall = Ml + nw * kQT * 2;
@@ -259,7 +307,7 @@ __global__ __launch_bounds__(512) void capped_attention_kernel(
 #pragma unroll
     for (int b = 0; b < NVB; ++b)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) Os[qi * ostride + b * 32 + 8 * (r / 4) + 4 * hl + (r % 4)] = o[b][r] * inv;
+      for (int r = 0; r < 16; ++r) Os[qi * ostride + (8 * (r / 4) + 4 * hl + (r % 4)) * NB + b] = o[b][r] * inv;
   }
   __syncthreads();
   if (!live) return;
@@ -274,7 +322,7 @@ __global__ __launch_bounds__(512) void capped_attention_kernel(
   }
 }
 
-template <typename T, int NVB>
+template <typename T, int NB>
 int launch_capped_attention(void* out, const float* q, const void* key_cache, const void* value_cache, const void* gate,
                             int64_t gate_stride, const int32_t* block_tables, int table_width, const int32_t* q_start,
                             const int32_t* ctx_len, int64_t rows, int num_seqs, int max_query_len, int heads,
@@ -282,7 +330,7 @@ int launch_capped_attention(void* out, const float* q, const void* key_cache, co
                             hipStream_t stream) {
   const int R = heads / kv_heads;
   const int tpt = kQT / R;
-  const int qstride = (dim + 31) / 32 * 32 + 4, ostride = NVB * 32 + 1;
+  const int qstride = (dim + 31) / 32 * 32 + 4, ostride = NB * 32 + 1;
   const bool split = max_query_len > 0 && max_query_len <= tpt;
   const int rows_used = split ? max_query_len * R : kQT;
   auto lds_bytes = [&](int nw) {
@@ -295,7 +343,10 @@ int launch_capped_attention(void* out, const float* q, const void* key_cache, co
   while (nw > 1 && lds_bytes(nw) > 72 * 1024) nw >>= 1;
   SW_CHECK_ARG(lds_bytes(nw) <= 160 * 1024, "capped_attention: key size %d with value size %d needs too much LDS", dim,
                vdim);
-  auto kernel = capped_attention_kernel<T, NVB>;
+  auto kernel = capped_attention_kernel<T, NB>;
+  int page_shift = -1;
+  if ((page_size & (page_size - 1)) == 0)
+    for (page_shift = 0; (1 << page_shift) < page_size; ++page_shift) {}
   static size_t allowed = 0;                                 // per instantiation
   if (lds_bytes(nw) > allowed) {
     SW_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -306,7 +357,7 @@ int launch_capped_attention(void* out, const float* q, const void* key_cache, co
   const dim3 grid((unsigned)(split ? tiles : (tiles + nw - 1) / nw), (unsigned)kv_heads);
   hipLaunchKernelGGL(kernel, grid, dim3(64 * nw), lds_bytes(nw), stream, out, q, key_cache, value_cache, gate,
                      gate_stride, block_tables, table_width, q_start, ctx_len, num_seqs, heads, kv_heads, dim, vdim,
-                     page_size, scale, softcap, window, tpt, split ? 1 : 0, rows_used);
+                     page_size, scale, softcap, window, tpt, split ? 1 : 0, rows_used, page_shift);
   SW_CHECK_LAUNCH();
   return SW_OK;
 }
@@ -324,9 +375,10 @@ extern "C" int swm_capped_attention(void* out, const float* q, const void* key_c
   SW_CHECK_ARG(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && heads / kv_heads <= kQT,
                "capped_attention: %d query heads on %d key/value heads (at most %d per key/value head)", heads, kv_heads,
                kQT);
-  SW_CHECK_ARG(dim > 0 && vdim > 0 && vdim <= 256 && page_size > 0 && table_width > 0 && rows < (1ll << 31),
-               "capped_attention: key size %d, value size %d (at most 256)", dim, vdim);
-  const int nvb = (vdim + 31) / 32;
+  SW_CHECK_ARG(dim > 0 && dim <= 256 && vdim > 0 && vdim <= 256 && page_size > 0 && table_width > 0 &&
+                   rows < (1ll << 31),
+               "capped_attention: key size %d, value size %d (at most 256 each)", dim, vdim);
+  const int nvb = std::max((vdim + 31) / 32, (dim + 31) / 32);
   hipStream_t s = static_cast<hipStream_t>(stream);
 #define SWM_CAPPED_CASE(N)                                                                                              \
   case N:                                                                                                               \

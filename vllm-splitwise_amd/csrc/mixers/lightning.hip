@@ -19,8 +19,9 @@ namespace swm {
 
 using f32x16 = __attribute__((ext_vector_type(16))) float;
 constexpr int kChunk = 32;
+constexpr int kWhole = 0, kLocal = 1, kFinal = 2;
+constexpr int kSegment = 128;          // tokens per segment of a long run (a multiple of kChunk)
 
-__device__ __forceinline__ float siluf_(float x) { return x / (1.0f + expf(-x)); }
 
 // NDB: 32-coordinate blocks of the key size.  A workgroup owns (sequence, head) and up to 8 blocks of 32 value
 // channels, one wave each; the chunk's silu(q) and silu(k) are staged once in LDS for all of them.
@@ -28,17 +29,31 @@ template <typename T, int NDB>
 __global__ __launch_bounds__(512) void lightning_kernel(
     float* __restrict__ out, const void* __restrict__ q, const void* __restrict__ k, const void* __restrict__ v,
     int64_t in_stride, const float* __restrict__ decay, float* __restrict__ state, const int32_t* __restrict__ q_start,
-    const int32_t* __restrict__ ctx_len, const int32_t* __restrict__ state_slot, int heads, int dim, int vdim) {
+    const int32_t* __restrict__ ctx_len, const int32_t* __restrict__ state_slot, int num_seqs, int heads, int dim,
+    int vdim, int mode, int seg_len, float* __restrict__ seg_state) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   constexpr int DS = NDB * 32 + 4;                           // row stride of the staged tiles
   float* Qs = lds;                                           // [32][DS]
   float* Ks = Qs + kChunk * DS;                              // [32][DS]
   float* pw = Ks + kChunk * DS;                              // [kChunk + 1] powers of the decay
-  const int seq = blockIdx.x, h = blockIdx.y;
+  const int h = blockIdx.y;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, li = lane & 31, hl = lane >> 5;
   const int vb = blockIdx.z * (blockDim.x >> 6) + wave;
-  const int row0 = q_start[seq], n = q_start[seq + 1] - row0;
+  // mode 0: blockIdx.x is a sequence and its whole run is taken from the slot's state to the slot's state.
+  // Long runs are cut into segments of seg_len tokens that run side by side: mode 1 takes every segment but a
+  // sequence's last from the EMPTY state and leaves its end state in seg_state[segment]; a scan (below) turns these
+  // into the states at the segments' ends; mode 2 then takes every segment from its true start state (the slot's for
+  // a sequence's first segment), writes the outputs, and a sequence's last segment leaves its state in the slot.
+  int seq = blockIdx.x, tok0 = 0, n;
+  if (mode == kWhole) {
+    n = q_start[seq + 1] - q_start[seq];
+  } else {
+    n = find_query_tile(q_start, num_seqs, blockIdx.x, seg_len, &seq, &tok0);
+  }
   if (n <= 0) return;                                        // the whole workgroup
+  const int row0 = q_start[seq] + tok0;
+  const bool last_seg = tok0 + n == q_start[seq + 1] - q_start[seq];
+  if (mode == kLocal && last_seg) return;
   const float lam = decay[h];
   if (threadIdx.x == 0) {
     float p = 1.0f;
@@ -51,14 +66,17 @@ __global__ __launch_bounds__(512) void lightning_kernel(
   const bool vc_ok = vc < vdim;
   float* sp = state + ((int64_t)state_slot[seq] * heads + h) * (int64_t)dim * vdim;
 
+  float* seg_out = seg_state + ((int64_t)blockIdx.x * heads + h) * (int64_t)dim * vdim;      // modes 1, 2 only
+  const float* start = (mode == kFinal && tok0 > 0) ? seg_out - (int64_t)heads * dim * vdim : sp;
+
   f32x16 S[NDB];
-  const bool fresh = ctx_len[seq] == 0;
+  const bool fresh = mode == kLocal || (tok0 == 0 && ctx_len[seq] == 0);
 #pragma unroll
   for (int b = 0; b < NDB; ++b)
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int c = 32 * b + 8 * (r / 4) + 4 * hl + (r % 4);
-      S[b][r] = (!fresh && vc_ok && c < dim) ? sp[(int64_t)c * vdim + vc] : 0.0f;
+      S[b][r] = (!fresh && vc_ok && c < dim) ? start[(int64_t)c * vdim + vc] : 0.0f;
     }
 
   const int64_t qk_col = (int64_t)h * dim, v_col = (int64_t)h * vdim;
@@ -70,8 +88,8 @@ __global__ __launch_bounds__(512) void lightning_kernel(
       const int r = e / (NDB * 32), c = e % (NDB * 32);
       float qv = 0.0f, kv = 0.0f;
       if (r < cn && c < dim) {
-        qv = siluf_(ld<T>(q, base + r * in_stride + qk_col + c));
-        kv = siluf_(ld<T>(k, base + r * in_stride + qk_col + c));
+        qv = fast_siluf_(ld<T>(q, base + r * in_stride + qk_col + c));
+        kv = fast_siluf_(ld<T>(k, base + r * in_stride + qk_col + c));
       }
       Qs[r * DS + c] = qv;
       Ks[r * DS + c] = kv;
@@ -81,7 +99,7 @@ __global__ __launch_bounds__(512) void lightning_kernel(
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int j = 8 * (r / 4) + 4 * hl + (r % 4);
-      vt[r] = (vc_ok && j < cn) ? siluf_(ld<T>(v, base + j * in_stride + v_col + vc)) : 0.0f;
+      vt[r] = (vc_ok && j < cn) ? fast_siluf_(ld<T>(v, base + j * in_stride + v_col + vc)) : 0.0f;
     }
     __syncthreads();
     // ---- A^T = K Q^T (rows: keys, columns: queries); this lane: token li of the chunk as key and as query
@@ -129,7 +147,7 @@ __global__ __launch_bounds__(512) void lightning_kernel(
         }
       }
     }
-    if (li < cn && vb * 32 < vdim) {
+    if (mode != kLocal && li < cn && vb * 32 < vdim) {
       float* dst = out + (int64_t)(row0 + c0 + li) * heads * vdim + v_col + vb * 32;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
@@ -153,21 +171,50 @@ __global__ __launch_bounds__(512) void lightning_kernel(
       }
     }
   }
+  if (mode == kFinal && !last_seg) return;                  // its end state is the next segment's start: known already
+  float* end = mode == kLocal ? seg_out : sp;
   if (vc_ok) {
 #pragma unroll
     for (int b = 0; b < NDB; ++b)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int c = 32 * b + 8 * (r / 4) + 4 * hl + (r % 4);
-        if (c < dim) sp[(int64_t)c * vdim + vc] = S[b][r];
+        if (c < dim) end[(int64_t)c * vdim + vc] = S[b][r];
       }
+  }
+}
+
+// seg_state[segment] (its end state from the empty state) -> the state at the segment's end:
+// S_end(j) = decay^seg_len S_end(j - 1) + local(j), S_end(-1) = the slot's state (nothing for a new sequence)
+__global__ __launch_bounds__(256) void lightning_scan_kernel(
+    float* __restrict__ seg_state, const float* __restrict__ state, const float* __restrict__ decay,
+    const int32_t* __restrict__ q_start, const int32_t* __restrict__ ctx_len, const int32_t* __restrict__ state_slot,
+    int heads, int dim, int vdim, int seg_len) {
+  const int seq = blockIdx.x, h = blockIdx.y;
+  const int e = blockIdx.z * 256 + threadIdx.x;
+  const int size = dim * vdim;
+  if (e >= size) return;
+  const int n = q_start[seq + 1] - q_start[seq];
+  const int segs = (n + seg_len - 1) / seg_len;
+  if (segs <= 1) return;
+  int first = 0;
+  for (int s = 0; s < seq; ++s) first += (q_start[s + 1] - q_start[s] + seg_len - 1) / seg_len;
+  float keep = 1.0f;
+  const float lam = decay[h];
+  for (int i = 0; i < seg_len; ++i) keep *= lam;
+  float S = ctx_len[seq] == 0 ? 0.0f : state[((int64_t)state_slot[seq] * heads + h) * size + e];
+  for (int j = 0; j + 1 < segs; ++j) {
+    float* p = seg_state + ((int64_t)(first + j) * heads + h) * size + e;
+    S = keep * S + *p;
+    *p = S;
   }
 }
 
 template <typename T, int NDB>
 int launch_lightning(float* out, const void* q, const void* k, const void* v, int64_t in_stride, const float* decay,
                      float* state, const int32_t* q_start, const int32_t* ctx_len, const int32_t* state_slot,
-                     int num_seqs, int heads, int dim, int vdim, hipStream_t stream) {
+                     int64_t rows, int num_seqs, int max_query_len, int heads, int dim, int vdim, float* seg_state,
+                     hipStream_t stream) {
   const int vblocks = (vdim + 31) / 32;
   const int waves = std::min(vblocks, 8);
   const size_t lds_bytes = (size_t)(2 * kChunk * (NDB * 32 + 4) + kChunk + 2) * sizeof(float);
@@ -178,19 +225,42 @@ int launch_lightning(float* out, const void* q, const void* k, const void* v, in
                                      (int)lds_bytes));
     raised = true;
   }
-  const dim3 grid((unsigned)num_seqs, (unsigned)heads, (unsigned)((vblocks + waves - 1) / waves));
-  hipLaunchKernelGGL(kernel, grid, dim3(64 * waves), lds_bytes, stream, out, q, k, v, in_stride, decay, state, q_start,
-                     ctx_len, state_slot, heads, dim, vdim);
+  const unsigned zgroups = (unsigned)((vblocks + waves - 1) / waves);
+  if (seg_state == nullptr || max_query_len <= 2 * kSegment) {
+    hipLaunchKernelGGL(kernel, dim3((unsigned)num_seqs, (unsigned)heads, zgroups), dim3(64 * waves), lds_bytes, stream,
+                       out, q, k, v, in_stride, decay, state, q_start, ctx_len, state_slot, num_seqs, heads, dim, vdim,
+                       kWhole, kSegment, seg_state);
+    SW_CHECK_LAUNCH();
+    return SW_OK;
+  }
+  const unsigned items = (unsigned)(rows / kSegment + num_seqs);
+  hipLaunchKernelGGL(kernel, dim3(items, (unsigned)heads, zgroups), dim3(64 * waves), lds_bytes, stream, out, q, k, v,
+                     in_stride, decay, state, q_start, ctx_len, state_slot, num_seqs, heads, dim, vdim, kLocal, kSegment,
+                     seg_state);
+  SW_CHECK_LAUNCH();
+  hipLaunchKernelGGL(lightning_scan_kernel, dim3((unsigned)num_seqs, (unsigned)heads, (unsigned)((dim * vdim + 255) / 256)),
+                     dim3(256), 0, stream, seg_state, state, decay, q_start, ctx_len, state_slot, heads, dim, vdim,
+                     kSegment);
+  SW_CHECK_LAUNCH();
+  hipLaunchKernelGGL(kernel, dim3(items, (unsigned)heads, zgroups), dim3(64 * waves), lds_bytes, stream, out, q, k, v,
+                     in_stride, decay, state, q_start, ctx_len, state_slot, num_seqs, heads, dim, vdim, kFinal, kSegment,
+                     seg_state);
   SW_CHECK_LAUNCH();
   return SW_OK;
 }
 
 }  // namespace swm
 
+extern "C" int64_t swm_lightning_workspace_floats(int64_t rows, int num_seqs, int max_query_len, int heads, int dim,
+                                                  int vdim) {
+  if (max_query_len <= 2 * swm::kSegment) return 0;
+  return (rows / swm::kSegment + num_seqs) * (int64_t)heads * dim * vdim;
+}
+
 extern "C" int swm_lightning(float* out, const void* q, const void* k, const void* v, int64_t in_stride,
                              const float* decay, float* state, const int32_t* q_start, const int32_t* ctx_len,
-                             const int32_t* state_slot, int64_t rows, int num_seqs, int heads, int dim, int vdim,
-                             int act_dtype, void* stream) {
+                             const int32_t* state_slot, int64_t rows, int num_seqs, int max_query_len, int heads,
+                             int dim, int vdim, float* workspace, int act_dtype, void* stream) {
   using namespace swm;
   if (rows == 0 || num_seqs == 0) return SW_OK;
   SW_CHECK_ARG(act_ok(act_dtype), "lightning: unsupported dtype %d", act_dtype);
@@ -200,7 +270,8 @@ extern "C" int swm_lightning(float* out, const void* q, const void* k, const voi
 #define SWM_LIGHTNING_CASE(N)                                                                                       \
   case N:                                                                                                           \
     SWM_DISPATCH_ACT(act_dtype, return (launch_lightning<T, N>(out, q, k, v, in_stride, decay, state, q_start,      \
-                                                               ctx_len, state_slot, num_seqs, heads, dim, vdim, s));); \
+                                                               ctx_len, state_slot, rows, num_seqs, max_query_len,  \
+                                                               heads, dim, vdim, workspace, s)););                  \
     break;
   switch ((dim + 31) / 32) {
     SWM_LIGHTNING_CASE(1)

@@ -24,6 +24,15 @@ __device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + expf
 // softplus without overflow: log(1 + e^x) = max(x, 0) + log1p(e^-|x|)
 __device__ __forceinline__ float softplusf_(float x) { return fmaxf(x, 0.0f) + log1pf(expf(-fabsf(x))); }
 
+// exp, sigmoid-weighted unit and tanh on the hardware's exp2 and reciprocal (a few ulp; for the inner loops of kernels
+// whose arithmetic is otherwise bound by these functions)
+__device__ __forceinline__ float fast_expf_(float x) { return __builtin_amdgcn_exp2f(x * 1.4426950408889634f); }
+__device__ __forceinline__ float fast_siluf_(float x) { return x * __builtin_amdgcn_rcpf(1.0f + fast_expf_(-x)); }
+// tanh(x) = 1 - 2 / (1 + e^(2x)); e^(2x) -> inf gives 1, -> 0 gives -1
+__device__ __forceinline__ float fast_tanhf_(float x) {
+  return 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + fast_expf_(2.0f * x));
+}
+
 // sum over the threads of a workgroup (blockDim.x a multiple of 64, at most 1024); every thread gets it
 __device__ __forceinline__ float block_sum(float v, float* lds /* >= 16 floats */) {
   v = sw::wave_sum(v);
@@ -34,6 +43,23 @@ __device__ __forceinline__ float block_sum(float v, float* lds /* >= 16 floats *
   float total = 0.0f;
   for (int w = 0; w < waves; ++w) total += lds[w];
   return total;
+}
+
+// -> sequence and first new token of tile `tile` when every sequence's new tokens are cut into runs of `tpt`;
+//    returns the tokens in the tile (0: no such tile)
+__device__ __forceinline__ int find_query_tile(const int32_t* __restrict__ q_start, int num_seqs, int tile, int tpt,
+                                               int* seq, int* tok0) {
+  for (int s = 0; s < num_seqs; ++s) {
+    const int n = q_start[s + 1] - q_start[s];
+    const int tiles = (n + tpt - 1) / tpt;
+    if (tile < tiles) {
+      *seq = s;
+      *tok0 = tile * tpt;
+      return min(tpt, n - tile * tpt);
+    }
+    tile -= tiles;
+  }
+  return 0;
 }
 
 }  // namespace swm

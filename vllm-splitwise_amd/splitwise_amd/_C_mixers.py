@@ -46,7 +46,7 @@ _SIGNATURES = {
     "swm_group_router": [_p, _p, _p, _p, _l, _i, _i, _i, _i, _f, _p],
     "swm_capped_attention": [_p, _p, _p, _p, _p, _l, _p, _i, _p, _p, _l, _i, _i, _i, _i, _i, _i, _i, _f, _f, _i, _i,
                              _p],
-    "swm_lightning": [_p, _p, _p, _p, _l, _p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p],
+    "swm_lightning": [_p, _p, _p, _p, _l, _p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p, _i, _p],
 }
 ACT_GELU, ACT_RELU2 = 0, 1
 
@@ -72,6 +72,8 @@ def load_library() -> ctypes.CDLL:
     lib = ctypes.CDLL(_LIB_PATH)
     lib.swm_last_error.restype, lib.swm_last_error.argtypes = ctypes.c_char_p, []
     lib.swm_abi_version.restype, lib.swm_abi_version.argtypes = _i, []
+    lib.swm_lightning_workspace_floats.restype = _l
+    lib.swm_lightning_workspace_floats.argtypes = [_l, _i, _i, _i, _i, _i]
     if lib.swm_abi_version() != ABI_VERSION:
         raise RuntimeError(f"{_LIB_PATH} implements interface version {lib.swm_abi_version()}, this binding needs "
                            f"{ABI_VERSION}: rebuild it (`make -C vllm-splitwise_amd mixers`)")
@@ -511,11 +513,15 @@ def lightning(out: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tens
           and _rows(k, "k") == stride and _rows(v, "v") == stride and k.dtype == q.dtype and v.dtype == q.dtype
           and out.shape == (rows, heads * vdim) and decay.numel() == heads and state.shape[1:] == (heads, dim, vdim)
           and batch.max_state_slot < state.shape[0], "lightning: shapes")
+    longest = int(getattr(batch, "max_query_len", 0) or 0)
     with _on_device_of(q):
-        _check(load_library().swm_lightning(out.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), stride,
-                                            decay.data_ptr(), state.data_ptr(), batch.q_start.data_ptr(),
-                                            batch.ctx_len.data_ptr(), batch.state_slot.data_ptr(), rows, n, heads, dim,
-                                            vdim, _act(q), _stream(q)))
+        lib = load_library()
+        need = lib.swm_lightning_workspace_floats(rows, n, longest, heads, dim, vdim)
+        work = torch.empty(need, dtype=torch.float32, device=q.device) if need > 0 else None
+        _check(lib.swm_lightning(out.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), stride, decay.data_ptr(),
+                                 state.data_ptr(), batch.q_start.data_ptr(), batch.ctx_len.data_ptr(),
+                                 batch.state_slot.data_ptr(), rows, n, longest, heads, dim, vdim, _opt_ptr(work),
+                                 _act(q), _stream(q)))
 
 
 ops = SimpleNamespace(expert_ffn=expert_ffn, ACT_GELU=ACT_GELU, ACT_RELU2=ACT_RELU2,
