@@ -305,8 +305,9 @@ def test_group_routed_experts(E, top, ff, shared, groups, keep, width, dtype):
     shared_out, routed = layer(h.to(DEV))
     got = routed.cpu().double() + (shared_out.cpu().double() if shared_out is not None else 0.0)
     want = oracle.moe_ff(h.double(), {k: v.double() for k, v in w.items()}, mlp)
-    tol = dict(atol=2e-4, rtol=2e-4) if dtype == torch.float32 else dict(atol=6e-2, rtol=6e-2)
-    torch.testing.assert_close(got, want, **tol)
+    # bf16: the hidden layer is rounded once and squared; errors are judged against the outputs' size
+    tol = 2e-5 if dtype == torch.float32 else 3e-2
+    assert (got - want).abs().max() < tol * want.abs().max()
 
 
 # --------------------------------------------------------------- whole models through the engine

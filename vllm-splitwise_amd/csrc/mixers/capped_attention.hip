@@ -168,38 +168,39 @@ __global__ __launch_bounds__(512) void capped_attention_kernel(
     if (page_shift >= 0) return (table[key >> page_shift] << page_shift) + (key & (page_size - 1));
     return table[key / page_size] * page_size + key % page_size;
   };
-  // all loads of one key tile: this lane's key row (runs of 16 per block) and the values of keys (r, hl)
-  auto issue = [&](int slot, Raw<T, 16> (&kraw)[NB], Raw<T, NB> (&vraw)[16]) {
+  // loads of one key tile: this lane's key row (runs of 16 per block); the values of keys (r, hl)
+  auto issue_keys = [&](int slot, Raw<T, 16> (&kraw)[NB]) {
     const int64_t krow = ((int64_t)max(slot, 0) * kv_heads + g) * dim;
 #pragma unroll
     for (int b = 0; b < NB; ++b)
       if (b < dblocks) load_raw(kraw[b], key_cache, krow, b * 32 + hl * 16, dim, slot >= 0, kvec);
+  };
+  auto issue_values = [&](int slot, Raw<T, NB> (&vraw)[16]) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int vslot = __shfl(slot, 8 * (r / 4) + 4 * hl + (r % 4), 64);
       load_raw(vraw[r], value_cache, ((int64_t)max(vslot, 0) * kv_heads + g) * vdim, qi * NB, vdim, vslot >= 0, vvec);
     }
   };
-  // small heads in a 16-bit cache: the next tile's loads are in flight while this tile's products run (two register
-  // sets); otherwise there are registers for one set only, and the next tile is loaded after the products
-  constexpr bool kAhead = sizeof(typename Conv<T>::store_t) == 2 && NB <= 2;
+  // A tile's values are asked for before its first product and arrive while it runs.  With a 16-bit cache and heads of
+  // up to 128 there are registers for a second set of keys: the NEXT tile's keys are asked for at the same time and
+  // arrive during this tile; otherwise a tile's keys are asked for when the tile before it ends.
+  constexpr bool kAhead = sizeof(typename Conv<T>::store_t) == 2 && NB <= 4;
   int kt = tile_lo + (split ? wave : 0);
   Raw<T, 16> kraw[NB];
-  Raw<T, NB> vraw[16];
-  int slot_next = -1;
+  int slot_cur = -1, slot_next = -1;
   if (kt <= tile_hi) {
-    issue(slot_of(kt * kQT), kraw, vraw);
+    slot_cur = slot_of(kt * kQT);
+    issue_keys(slot_cur, kraw);
     if (kt + kstep <= tile_hi) slot_next = slot_of((kt + kstep) * kQT);
   }
   for (; kt <= tile_hi; kt += kstep) {
     const int k0 = kt * kQT;
+    Raw<T, NB> vraw[16];
+    issue_values(slot_cur, vraw);
     Raw<T, 16> kraw2[NB];
-    Raw<T, NB> vraw2[16];
-    int slot_next2 = -1;
-    if (kAhead) {
-      if (kt + kstep <= tile_hi) issue(slot_next, kraw2, vraw2);
-      if (kt + 2 * kstep <= tile_hi) slot_next2 = slot_of((kt + 2 * kstep) * kQT);
-    }
+    if (kAhead && kt + kstep <= tile_hi) issue_keys(slot_next, kraw2);
+    const int slot_next2 = kt + 2 * kstep <= tile_hi ? slot_of((kt + 2 * kstep) * kQT) : -1;
     // ---- S^T = K Q^T
     f32x16 s;
 #pragma unroll
@@ -257,13 +258,11 @@ __global__ __launch_bounds__(512) void capped_attention_kernel(
     if (kAhead) {
 #pragma unroll
       for (int b = 0; b < NB; ++b) kraw[b] = kraw2[b];
-#pragma unroll
-      for (int r = 0; r < 16; ++r) vraw[r] = vraw2[r];
-      slot_next = slot_next2;
     } else if (kt + kstep <= tile_hi) {
-      issue(slot_next, kraw, vraw);
-      slot_next = kt + 2 * kstep <= tile_hi ? slot_of((kt + 2 * kstep) * kQT) : -1;
+      issue_keys(slot_next, kraw);
     }
+    slot_cur = slot_next;
+    slot_next = slot_next2;
   }
 
   if (split) {
