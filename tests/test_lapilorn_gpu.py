@@ -162,7 +162,7 @@ def _paged(k, v, G, d, dv, page, dtype, seed):
 
 @pytest.mark.parametrize("H,G,d,dv,page", [(4, 2, 16, 32, 16), (6, 6, 8, 8, 16), (3, 1, 24, 72, 8), (8, 2, 20, 40, 16),
                                            (2, 1, 128, 128, 64), (5, 1, 12, 130, 16), (4, 4, 64, 16, 32)])
-@pytest.mark.parametrize("mode", ["prompt", "decode", "portions"])
+@pytest.mark.parametrize("mode", ["prompt", "decode", "pairs", "portions"])
 @pytest.mark.parametrize("cache_dtype,cap,window", [(torch.float32, 5.0, 0), (torch.bfloat16, 5.0, 0), (torch.float32, 0.0, 0),
                                                     (torch.float32, 5.0, 37)])
 def test_capped_attention_edges(H, G, d, dv, page, mode, cache_dtype, cap, window):
@@ -187,6 +187,10 @@ def test_capped_attention_edges(H, G, d, dv, page, mode, cache_dtype, cap, windo
     elif mode == "decode":
         rows = list(range(n - 45, n)) + [0, 1, 33]
         seqs = [(t, 1, 0, table) for t in rows]
+    elif mode == "pairs":                                             # steps of two tokens, and one of a single token
+        firsts = list(range(n - 46, n, 2)) + [0, 32, 127]
+        seqs = [(t, 2, 0, table) for t in firsts] + [(n - 47, 1, 0, table)]
+        rows = [t + i for t in firsts for i in range(2)] + [n - 47]
     else:
         cuts, at = [], 0
         for size in [3, 2, 27, 1, 31, 2, 64, 2, 33, 5, 32, 98]:

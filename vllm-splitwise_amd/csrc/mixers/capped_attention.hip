@@ -321,6 +321,191 @@ __global__ __launch_bounds__(512) void capped_attention_kernel(
   }
 }
 
+// Steps of very few query rows per sequence and key/value head (a decode step: one token's R query heads) leave a
+// 32-row matrix tile mostly empty, so they run on the vector units instead: LK (8 or 16) lanes share a key, each with C
+// coordinates of the key, of every query row and of the value; a wave walks 64 / LK keys at a time, a workgroup owns
+// (sequence, key/value head).  Every lane group keeps a running softmax of its own; groups are joined by shuffles,
+// waves through LDS, both in a fixed order.  RQ: query rows (padded), C: coordinates per lane, U: keys in flight.
+template <typename T, int RQ, int C, int LK, int U>
+__global__ __launch_bounds__(512) void capped_attention_rows_kernel(
+    void* __restrict__ out, const float* __restrict__ q, const void* __restrict__ key_cache,
+    const void* __restrict__ value_cache, const void* __restrict__ gate, int64_t gate_stride,
+    const int32_t* __restrict__ block_tables, int table_width, const int32_t* __restrict__ q_start,
+    const int32_t* __restrict__ ctx_len, int heads, int kv_heads, int dim, int vdim, int page_size, int page_shift,
+    float scale, float softcap, int window) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  const int seq = blockIdx.x, g = blockIdx.y, R = heads / kv_heads;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, pt = lane % LK, grp = lane / LK, nw = blockDim.x >> 6;
+  const int row0 = q_start[seq], n = q_start[seq + 1] - row0;
+  if (n <= 0) return;                                        // the whole workgroup
+  const int ctx = ctx_len[seq], rows = n * R, last_pos = ctx + n - 1;
+  const int32_t* table = block_tables + (int64_t)seq * table_width;
+  float* Ml = lds;                                           // [nw][RQ][2]
+  float* Os = lds + nw * RQ * 2;                             // [nw][RQ][LK * C]
+
+  float qv[RQ][C], o[RQ][C], m_run[RQ], l_run[RQ];
+  int pos[RQ];
+#pragma unroll
+  for (int r = 0; r < RQ; ++r) {
+    const int tt = r / R, hh = r % R;
+    pos[r] = ctx + min(tt, n - 1);                           // padding rows behave like the last token's
+    m_run[r] = -INFINITY;
+    l_run[r] = 0.0f;
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+      const int col = pt * C + c;
+      qv[r][c] = (r < rows && col < dim) ? q[(int64_t)(row0 + tt) * heads * dim + (int64_t)(g * R + hh) * dim + col] * scale
+                                         : 0.0f;
+      o[r][c] = 0.0f;
+    }
+  }
+  const bool kvec = dim % (C >= 8 ? 8 : 4) == 0, vvec = vdim % (C >= 8 ? 8 : 4) == 0;
+  const float inv_cap = softcap > 0.0f ? 1.0f / softcap : 0.0f;
+  const int lowest = window > 0 ? max(0, ctx - window + 1) : 0;
+  constexpr int GW = 64 / LK;                                // lane groups of a wave
+  const int groups = nw * GW;
+  for (int key0 = lowest + wave * GW + grp; key0 <= last_pos; key0 += groups * U) {
+    Raw<T, C> kr[U], vr[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int key = key0 + u * groups;
+      const bool ok = key <= last_pos;
+      int slot = 0;
+      if (ok) slot = page_shift >= 0 ? (table[key >> page_shift] << page_shift) + (key & (page_size - 1))
+                                     : table[key / page_size] * page_size + key % page_size;
+      load_raw(kr[u], key_cache, ((int64_t)slot * kv_heads + g) * dim, pt * C, dim, ok, kvec);
+      load_raw(vr[u], value_cache, ((int64_t)slot * kv_heads + g) * vdim, pt * C, vdim, ok, vvec);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int key = key0 + u * groups;
+      if (key > last_pos) continue;                          // uniform over the lane group
+#pragma unroll
+      for (int r = 0; r < RQ; ++r) {
+        float s = 0.0f;
+#pragma unroll
+        for (int c = 0; c < C; ++c) s += qv[r][c] * kr[u].get(c);
+        s = lanes_sum<LK>(s);
+        if (softcap > 0.0f) s = softcap * fast_tanhf_(s * inv_cap);
+        const bool seen = key <= pos[r] && (window <= 0 || pos[r] - key < window);
+        if (!seen) s = -INFINITY;
+        const float m_new = fmaxf(m_run[r], s);
+        const float m_use = m_new == -INFINITY ? 0.0f : m_new;
+        const float alpha = fast_expf_(m_run[r] - m_use);
+        const float p = fast_expf_(s - m_use);
+        l_run[r] = l_run[r] * alpha + p;
+        m_run[r] = m_new;
+#pragma unroll
+        for (int c = 0; c < C; ++c) o[r][c] = o[r][c] * alpha + p * vr[u].get(c);
+      }
+    }
+  }
+  // ---- join the wave's lane groups
+#pragma unroll
+  for (int step = LK; step <= 32; step <<= 1) {
+#pragma unroll
+    for (int r = 0; r < RQ; ++r) {
+      const float m_o = __shfl_xor(m_run[r], step, 64), l_o = __shfl_xor(l_run[r], step, 64);
+      const float m_new = fmaxf(m_run[r], m_o);
+      const float m_use = m_new == -INFINITY ? 0.0f : m_new;
+      const float fa = fast_expf_(m_run[r] - m_use), fb = fast_expf_(m_o - m_use);
+      l_run[r] = l_run[r] * fa + l_o * fb;
+      m_run[r] = m_new;
+#pragma unroll
+      for (int c = 0; c < C; ++c) o[r][c] = o[r][c] * fa + __shfl_xor(o[r][c], step, 64) * fb;
+    }
+  }
+  // ---- join the waves
+  if (grp == 0) {
+#pragma unroll
+    for (int r = 0; r < RQ; ++r) {
+      if (pt == 0) {
+        Ml[(wave * RQ + r) * 2] = m_run[r];
+        Ml[(wave * RQ + r) * 2 + 1] = l_run[r];
+      }
+#pragma unroll
+      for (int c = 0; c < C; ++c) Os[(wave * RQ + r) * LK * C + pt * C + c] = o[r][c];
+    }
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < rows * vdim; e += blockDim.x) {
+    const int r = e / vdim, c = e % vdim;
+    const int tt = r / R, hh = r % R;
+    float m_all = -INFINITY;
+    for (int w = 0; w < nw; ++w) m_all = fmaxf(m_all, Ml[(w * RQ + r) * 2]);
+    float num = 0.0f, den = 0.0f;
+    for (int w = 0; w < nw; ++w) {
+      const float f = fast_expf_(Ml[(w * RQ + r) * 2] - m_all);      // a wave that saw no key: 0
+      den += f * Ml[(w * RQ + r) * 2 + 1];
+      num += f * Os[(w * RQ + r) * LK * C + c];
+    }
+    float v = num / den;
+    const int64_t col = (int64_t)(g * R + hh) * vdim + c;
+    if (gate != nullptr) v *= sigmoidf_(ld<T>(gate, (row0 + tt) * gate_stride + col));
+    st<T>(out, (int64_t)(row0 + tt) * heads * vdim + col, v);
+  }
+}
+
+template <typename T, int RQ, int C, int LK>
+int launch_capped_rows(void* out, const float* q, const void* key_cache, const void* value_cache, const void* gate,
+                       int64_t gate_stride, const int32_t* block_tables, int table_width, const int32_t* q_start,
+                       const int32_t* ctx_len, int num_seqs, int heads, int kv_heads, int dim, int vdim, int page_size,
+                       float scale, float softcap, int window, hipStream_t stream) {
+  constexpr bool half = sizeof(typename Conv<T>::store_t) == 2;
+  constexpr int U = RQ * C <= 32 ? (half ? 4 : 2) : (half ? 2 : 1);
+  const int nw = 8;
+  const size_t lds_bytes = (size_t)nw * RQ * (2 + LK * C) * sizeof(float);
+  int page_shift = -1;
+  if ((page_size & (page_size - 1)) == 0)
+    for (page_shift = 0; (1 << page_shift) < page_size; ++page_shift) {}
+  auto kernel = capped_attention_rows_kernel<T, RQ, C, LK, U>;
+  static bool raised = false;                                // per instantiation
+  if (lds_bytes > 64 * 1024 && !raised) {
+    SW_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     (int)lds_bytes));
+    raised = true;
+  }
+  hipLaunchKernelGGL(kernel, dim3((unsigned)num_seqs, (unsigned)kv_heads), dim3(64 * nw), lds_bytes, stream, out, q,
+                     key_cache, value_cache, gate, gate_stride, block_tables, table_width, q_start, ctx_len, heads,
+                     kv_heads, dim, vdim, page_size, page_shift, scale, softcap, window);
+  SW_CHECK_LAUNCH();
+  return SW_OK;
+}
+
+// -> true when the step was taken by the vector-unit kernel (few rows, lanes' shares small enough for registers)
+template <typename T>
+bool try_capped_rows(int* status, int rows_used, void* out, const float* q, const void* key_cache,
+                     const void* value_cache, const void* gate, int64_t gate_stride, const int32_t* block_tables,
+                     int table_width, const int32_t* q_start, const int32_t* ctx_len, int num_seqs, int heads,
+                     int kv_heads, int dim, int vdim, int page_size, float scale, float softcap, int window,
+                     hipStream_t stream) {
+  if (rows_used > 8) return false;
+  auto pow2 = [](int x) { return x <= 4 ? 4 : x <= 8 ? 8 : x <= 16 ? 16 : x <= 32 ? 32 : 64; };
+  const int most = std::max(dim, vdim);
+  const int rq = rows_used <= 1 ? 1 : rows_used <= 2 ? 2 : rows_used <= 4 ? 4 : 8;
+  // 8 lanes per key while a lane's share of rows x coordinates stays small, else 16
+  int lk = 8, c = pow2((most + 7) / 8);
+  if (rq * c > 64) {
+    lk = 16;
+    c = pow2((most + 15) / 16);
+  }
+  if (rq * c > 64) return false;
+#define SWM_ROWS_CASE(RQV, CV, LKV)                                                                                     \
+  if (rq == RQV && c == CV && lk == LKV) {                                                                              \
+    *status = launch_capped_rows<T, RQV, CV, LKV>(out, q, key_cache, value_cache, gate, gate_stride, block_tables,      \
+                                                  table_width, q_start, ctx_len, num_seqs, heads, kv_heads, dim, vdim,  \
+                                                  page_size, scale, softcap, window, stream);                           \
+    return true;                                                                                                        \
+  }
+  SWM_ROWS_CASE(1, 4, 8) SWM_ROWS_CASE(1, 8, 8) SWM_ROWS_CASE(1, 16, 8) SWM_ROWS_CASE(1, 32, 8)
+  SWM_ROWS_CASE(2, 4, 8) SWM_ROWS_CASE(2, 8, 8) SWM_ROWS_CASE(2, 16, 8) SWM_ROWS_CASE(2, 32, 8)
+  SWM_ROWS_CASE(4, 4, 8) SWM_ROWS_CASE(4, 8, 8) SWM_ROWS_CASE(4, 16, 8)
+  SWM_ROWS_CASE(8, 4, 8) SWM_ROWS_CASE(8, 8, 8)
+  SWM_ROWS_CASE(4, 16, 16) SWM_ROWS_CASE(8, 8, 16)
+#undef SWM_ROWS_CASE
+  return false;
+}
+
 template <typename T, int NB>
 int launch_capped_attention(void* out, const float* q, const void* key_cache, const void* value_cache, const void* gate,
                             int64_t gate_stride, const int32_t* block_tables, int table_width, const int32_t* q_start,
@@ -332,6 +517,13 @@ int launch_capped_attention(void* out, const float* q, const void* key_cache, co
   const int qstride = (dim + 31) / 32 * 32 + 4, ostride = NB * 32 + 1;
   const bool split = max_query_len > 0 && max_query_len <= tpt;
   const int rows_used = split ? max_query_len * R : kQT;
+  if (split) {
+    int status = SW_OK;
+    if (try_capped_rows<T>(&status, rows_used, out, q, key_cache, value_cache, gate, gate_stride, block_tables, table_width,
+                           q_start, ctx_len, num_seqs, heads, kv_heads, dim, vdim, page_size, scale, softcap, window,
+                           stream))
+      return status;
+  }
   auto lds_bytes = [&](int nw) {
     const size_t floats = split ? (size_t)kQT * qstride + (size_t)nw * kQT * 2 + (size_t)nw * rows_used * ostride
                                 : (size_t)nw * kQT * std::max(qstride, ostride);

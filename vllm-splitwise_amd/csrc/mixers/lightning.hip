@@ -203,10 +203,20 @@ __global__ __launch_bounds__(256) void lightning_scan_kernel(
   const float lam = decay[h];
   for (int i = 0; i < seg_len; ++i) keep *= lam;
   float S = ctx_len[seq] == 0 ? 0.0f : state[((int64_t)state_slot[seq] * heads + h) * size + e];
-  for (int j = 0; j + 1 < segs; ++j) {
-    float* p = seg_state + ((int64_t)(first + j) * heads + h) * size + e;
-    S = keep * S + *p;
-    *p = S;
+  // eight segments at a time: their loads do not wait for one another
+  const int64_t stride = (int64_t)heads * size;
+  float* p = seg_state + ((int64_t)first * heads + h) * size + e;
+  for (int j0 = 0; j0 + 1 < segs; j0 += 8) {
+    float local[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) local[i] = j0 + i + 1 < segs ? p[(j0 + i) * stride] : 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (j0 + i + 1 < segs) {
+        S = keep * S + local[i];
+        p[(j0 + i) * stride] = S;
+      }
+    }
   }
 }
 

@@ -33,6 +33,22 @@ __device__ __forceinline__ float fast_tanhf_(float x) {
   return 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + fast_expf_(2.0f * x));
 }
 
+// sum over groups of LK = 8 or 16 neighbouring lanes (every lane of a group gets it): DPP quad permutes and row
+// mirrors, full-rate vector instructions with no trip through the LDS crossbar
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+template <int LK>
+__device__ __forceinline__ float lanes_sum(float v) {
+  static_assert(LK == 8 || LK == 16, "groups of 8 or 16 lanes");
+  v += dpp_move<0xB1>(v);                                    // quad_perm [1, 0, 3, 2]
+  v += dpp_move<0x4E>(v);                                    // quad_perm [2, 3, 0, 1]: every lane of a quad has the quad's sum
+  v += dpp_move<0x141>(v);                                   // row_half_mirror: lane i of 8 reads lane 7 - i, the other quad
+  if (LK == 16) v += dpp_move<0x140>(v);                     // row_mirror: lane i of 16 reads lane 15 - i, the other half
+  return v;
+}
+
 // sum over the threads of a workgroup (blockDim.x a multiple of 64, at most 1024); every thread gets it
 __device__ __forceinline__ float block_sum(float v, float* lds /* >= 16 floats */) {
   v = sw::wave_sum(v);
