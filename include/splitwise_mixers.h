@@ -175,6 +175,11 @@ int swm_rope_cache(float* q_out, const void* q, const void* k, const void* v, in
 int swm_group_router(int32_t* chosen, float* weights, const float* logits, const float* correction, int64_t rows,
                      int experts, int top, int groups, int keep, float scale, void* stream);
 
+/* chosen (int32 [pairs], every value in [0, experts)) -> order (int32 [pairs]: the pair indices grouped by expert) and
+ * expert_start (int32 [experts + 1]: every expert's first place in `order`); what the expert kernels take. */
+int swm_group_pairs(int32_t* order, int32_t* expert_start, const int32_t* chosen, int64_t pairs, int experts,
+                    void* stream);
+
 /* Causal softmax attention of every new token over its sequence's paged keys with grouped query heads (query head
  * h reads key/value head h / (heads / kv_heads)): score = (q . k) * scale, then softcap * tanh(score / softcap) when
  * softcap > 0; position i sees j <= i (and i - j < window when window > 0); fp32 scores, weights and sums.

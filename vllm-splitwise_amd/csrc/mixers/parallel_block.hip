@@ -178,6 +178,36 @@ __global__ __launch_bounds__(256) void group_router_kernel(
   for (int n = 0; n < top; ++n) weights[t * top + n] *= f;
 }
 
+
+// (row, choice) pairs grouped by expert in ONE launch of one workgroup: a histogram of the chosen experts in LDS, its
+// running sum = every expert's first sorted pair, then every pair takes the next place of its expert.  The order
+// inside an expert is whatever the LDS counters hand out: the experts' rows are independent, so it does not matter.
+constexpr int kPairThreads = 1024;
+
+__global__ __launch_bounds__(kPairThreads) void group_pairs_kernel(int32_t* __restrict__ order,
+                                                                   int32_t* __restrict__ expert_start,
+                                                                   const int32_t* __restrict__ chosen, int64_t pairs,
+                                                                   int experts) {
+  __shared__ int count[kMaxRouterExperts + 1];
+  __shared__ int cursor[kMaxRouterExperts];
+  for (int e = threadIdx.x; e <= experts; e += kPairThreads) count[e] = 0;
+  __syncthreads();
+  for (int64_t p = threadIdx.x; p < pairs; p += kPairThreads) atomicAdd(&count[chosen[p]], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int run = 0;
+    for (int e = 0; e < experts; ++e) {
+      const int n = count[e];
+      expert_start[e] = run;
+      cursor[e] = run;
+      run += n;
+    }
+    expert_start[experts] = run;
+  }
+  __syncthreads();
+  for (int64_t p = threadIdx.x; p < pairs; p += kPairThreads) order[atomicAdd(&cursor[chosen[p]], 1)] = (int32_t)p;
+}
+
 }  // namespace swm
 
 extern "C" {
@@ -254,6 +284,17 @@ int swm_group_router(int32_t* chosen, float* weights, const float* logits, const
                "group_router: %d groups, %d kept, %d experts, top %d", groups, keep, experts, top);
   hipLaunchKernelGGL(group_router_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, static_cast<hipStream_t>(stream),
                      chosen, weights, logits, correction, rows, experts, top, groups, keep, scale);
+  SW_CHECK_LAUNCH();
+  return SW_OK;
+}
+
+int swm_group_pairs(int32_t* order, int32_t* expert_start, const int32_t* chosen, int64_t pairs, int experts,
+                    void* stream) {
+  using namespace swm;
+  SW_CHECK_ARG(experts > 0 && experts <= kMaxRouterExperts && pairs >= 0 && pairs < (1ll << 31),
+               "group_pairs: %d experts (1..%d supported)", experts, kMaxRouterExperts);
+  hipLaunchKernelGGL(group_pairs_kernel, dim3(1), dim3(kPairThreads), 0, static_cast<hipStream_t>(stream), order,
+                     expert_start, chosen, pairs, experts);
   SW_CHECK_LAUNCH();
   return SW_OK;
 }

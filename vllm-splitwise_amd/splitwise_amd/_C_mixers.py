@@ -44,6 +44,7 @@ _SIGNATURES = {
     "swm_relu2": [_p, _p, _l, _l, _i, _i, _p],
     "swm_rope_cache": [_p, _p, _p, _p, _l, _p, _p, _i, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p],
     "swm_group_router": [_p, _p, _p, _p, _l, _i, _i, _i, _i, _f, _p],
+    "swm_group_pairs": [_p, _p, _p, _l, _i, _p],
     "swm_capped_attention": [_p, _p, _p, _p, _p, _l, _p, _i, _p, _p, _l, _i, _i, _i, _i, _i, _i, _i, _f, _f, _i, _i,
                              _p],
     "swm_lightning": [_p, _p, _p, _p, _l, _p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p, _i, _p],
@@ -470,6 +471,20 @@ def group_router(logits: torch.Tensor, correction: Optional[torch.Tensor], top: 
     return chosen, weights
 
 
+def group_pairs(chosen: torch.Tensor, experts: int):
+    """chosen int32 [rows, top] -> (order int32 [rows * top]: pair indices row * top + choice grouped by expert,
+    expert_start int32 [experts + 1]); one launch, nothing travels to the host."""
+    _dev(chosen)
+    _need(chosen.dtype == torch.int32 and chosen.is_contiguous(), "group_pairs: chosen must be contiguous int32")
+    pairs = chosen.numel()
+    order = torch.empty(pairs, dtype=torch.int32, device=chosen.device)
+    start = torch.empty(experts + 1, dtype=torch.int32, device=chosen.device)
+    with _on_device_of(chosen):
+        _check(load_library().swm_group_pairs(order.data_ptr(), start.data_ptr(), chosen.data_ptr(), pairs, experts,
+                                              _stream(chosen)))
+    return order, start
+
+
 def capped_attention(out: torch.Tensor, q: torch.Tensor, key_cache: torch.Tensor, value_cache: torch.Tensor,
                      gate: Optional[torch.Tensor], batch, heads: int, kv_heads: int, dim: int, vdim: int, scale: float,
                      softcap: float = 0.0, window: int = 0) -> None:
@@ -528,5 +543,5 @@ ops = SimpleNamespace(expert_ffn=expert_ffn, ACT_GELU=ACT_GELU, ACT_RELU2=ACT_RE
     scalar_norm_add=scalar_norm_add, scalar_norm=scalar_norm, qk_norm_cache=qk_norm_cache,
     window_attention=window_attention, short_conv=short_conv, channel_delta=channel_delta,
     general_delta=general_delta, head_norm_gate=head_norm_gate, stream_add_norm=stream_add_norm,
-    clamped_glu=clamped_glu, relu2=relu2, rope_cache=rope_cache, group_router=group_router,
+    clamped_glu=clamped_glu, relu2=relu2, rope_cache=rope_cache, group_router=group_router, group_pairs=group_pairs,
     capped_attention=capped_attention, lightning=lightning)

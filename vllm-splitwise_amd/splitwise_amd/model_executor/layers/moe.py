@@ -69,12 +69,9 @@ class TableRoutedExperts(nn.Module):
 
 
 def group_pairs_by_expert(experts: torch.Tensor, num_experts: int):
-    """experts int32 [rows, top] -> (order int32 [rows * top]: pair index row * top + choice sorted by expert,
-    expert_start int32 [experts + 1]); all on the device."""
-    flat = experts.reshape(-1)
-    by_expert, order = torch.sort(flat, stable=True)
-    edges = torch.arange(num_experts + 1, dtype=flat.dtype, device=flat.device)
-    return order.to(torch.int32), torch.searchsorted(by_expert, edges).to(torch.int32)
+    """experts int32 [rows, top] -> (order int32 [rows * top]: pair indices row * top + choice grouped by expert,
+    expert_start int32 [experts + 1]); one launch on the device."""
+    return _C.mixer_ops.group_pairs(experts, num_experts)
 
 
 class GroupRoutedExperts(nn.Module):
