@@ -91,7 +91,13 @@ def _check(status: int) -> None:
                            or f"splitwise_mixers call failed with status {status}")
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(t: torch.Tensor) -> int:
+    """torch's current HIP stream on ``t``'s device (the raw handle; a step makes a hundred of these calls)."""
+    if _raw_stream is not None:
+        return _raw_stream(t.device.index)
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
